@@ -1,0 +1,143 @@
+/*
+ * steptron_moe.h -- C ABI of libsteptron_moe_gfx950.so: hand-written HIP kernels
+ * (gfx950 / MI355X) for the MoE-layer hot path of StepTronOSS:
+ *   router -> permute -> routed grouped FFN (grouped GEMM + SwiGLU) -> unpermute.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its comment says "host";
+ *   - nothing here allocates, frees, synchronises with the host or throws: outputs
+ *     and scratch ("workspace") are passed in by the caller, sizes come from the
+ *     *_workspace_bytes() queries; all work is enqueued on `stream` (a hipStream_t);
+ *   - return value: STM_OK (0) or a negative STM_ERR_* code, see stm_status_string();
+ *   - matrices are row-major and dense unless a leading dimension is given;
+ *   - "ids": expert id per (token, k) slot, flat order token-major / k-minor; a
+ *     negative id marks an unused slot and is ignored everywhere;
+ *   - "pos": row of a slot in the expert-contiguous buffer (int32), negative = unused.
+ *
+ * Each entry point cites the reference interface it stands in for (paths relative to
+ * the StepTronOSS checkout).  The Python functions of the same name in
+ * steptronoss_amd/model/utils/moe_utils.py are thin callers of these.
+ */
+#ifndef STEPTRON_MOE_H_
+#define STEPTRON_MOE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* stm_stream_t; /* a hipStream_t; NULL = the default stream */
+
+/* element types */
+enum { STM_F32 = 0, STM_F16 = 1, STM_BF16 = 2 };
+
+/* status codes */
+enum {
+  STM_OK = 0,
+  STM_ERR_ARG = -1,         /* null pointer, negative size, inconsistent shapes   */
+  STM_ERR_UNSUPPORTED = -2, /* dtype / size outside what the kernels implement    */
+  STM_ERR_WORKSPACE = -3,   /* workspace smaller than *_workspace_bytes() said    */
+  STM_ERR_LAUNCH = -4       /* the HIP runtime refused the launch                 */
+};
+
+/* Device-side status words, int32[STM_STATUS_WORDS], written by the routing and
+ * index-check kernels with plain stores (a set word holds 1).  The caller zeroes the
+ * block when it wants a fresh reading and reads it back only if it wants to raise. */
+enum {
+  STM_ST_ID_OUT_OF_RANGE = 0, /* an id >= n_experts was seen (it is then ignored)         */
+  STM_ST_N_VALID = 1,         /* number of non-negative, in-range slots                   */
+  STM_ST_HIST_MISMATCH = 2,   /* sum(expert_histogram) != number of valid slots           */
+  STM_ST_HIST_NEGATIVE = 3,   /* expert_histogram has a negative entry                    */
+  STM_ST_NOT_INJECTIVE = 4,   /* two slots name the same row                              */
+  STM_ST_ROW_OUT_OF_RANGE = 5, /* a pos >= n_rows was seen                                 */
+  STM_ST_MAX_ROW_PLUS1 = 6,   /* 1 + the largest pos seen by stm_index_check (0 if none)  */
+  STM_STATUS_WORDS = 8
+};
+
+int stm_abi_version(void);
+const char* stm_status_string(int status);
+
+/* ------------------------------------------------------------------------------------
+ * Routing: per-expert histogram and stable counting-sort positions.
+ * Deterministic, no atomics: wave-level match/popcount ranks, per-wave LDS counters,
+ * one scan over (segment, expert).
+ * ---------------------------------------------------------------------------------- */
+
+/* Scratch needed by stm_histogram / stm_index_compute / stm_route_plan. */
+size_t stm_route_workspace_bytes(int64_t n_slots, int n_experts);
+
+/* histogram(top_k_rank, expert_num) -> int32 [E]
+ * replaces steptronoss/model/utils/moe_utils.py:90-129.
+ * status: int32[STM_STATUS_WORDS] device words (see STM_ST_*). */
+int stm_histogram(const void* ids, int ids_are_i64, int64_t n_slots, int n_experts, int32_t* hist_out,
+                  int32_t* status, void* workspace, size_t workspace_bytes, stm_stream_t stream);
+
+/* index_compute(indices, expert_histogram) -> int32 [T, K]
+ * replaces steptronoss/model/utils/moe_utils.py:137-214: pos = base[e] + stable rank of
+ * the slot among the slots of expert e, base = exclusive cumsum of the GIVEN histogram;
+ * negative ids are copied through. */
+int stm_index_compute(const void* ids, int ids_are_i64, int64_t n_slots, int n_experts, const void* hist_in,
+                      int hist_is_i64, int32_t* pos_out, int32_t* status, void* workspace, size_t workspace_bytes,
+                      stm_stream_t stream);
+
+/* Fused form used by routed_grouped_ffn (moe_utils.py:222-236): one call gives the
+ * histogram, the expert row offsets (int32 [E+1], offsets[E] = number of valid slots)
+ * and the positions, with no host round trip. */
+int stm_route_plan(const void* ids, int ids_are_i64, int64_t n_slots, int n_experts, int32_t* hist_out,
+                   int32_t* offsets_out, int32_t* pos_out, int32_t* status, void* workspace, size_t workspace_bytes,
+                   stm_stream_t stream);
+
+/* int64/int32 group sizes -> int32 offsets [G+1] (grouped_gemm's batch_sizes,
+ * moe_utils.py:443-453). */
+int stm_group_offsets(const void* sizes, int sizes_are_i64, int n_groups, int32_t* offsets_out, stm_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * Permute (reference name: moe_scatter) and unpermute (moe_weighted_gather).
+ * Pure row traffic: one workgroup per token, 128-bit accesses when rows allow.
+ * ---------------------------------------------------------------------------------- */
+
+/* MoEScatter.forward, moe_utils.py:339-374: out[pos[t,k], :] = x[t, :] for pos >= 0.
+ * Rows of `out` that no slot names are left untouched (see stm_zero_unwritten_rows).
+ * row_bytes = hidden * element size; any element type. */
+int stm_permute_fwd(const void* x, const void* pos, int pos_is_i64, void* out, int64_t n_tokens, int top_k,
+                    int64_t row_bytes, int64_t n_out_rows, uint8_t* written_or_null, stm_stream_t stream);
+
+/* Zero the rows r < n_out_rows with written[r] == 0 (the reference starts from
+ * new_zeros, moe_utils.py:356); only needed when pos is not a bijection. */
+int stm_zero_unwritten_rows(void* out, const uint8_t* written, int64_t n_out_rows, int64_t row_bytes,
+                            stm_stream_t stream);
+
+/* MoEScatter.backward, moe_utils.py:376-399: gx[t,:] = sum_k go[pos[t,k], :] over pos >= 0,
+ * accumulated in fp32 and rounded once. */
+int stm_permute_bwd(const void* grad_out, const void* pos, int pos_is_i64, void* grad_x, int64_t n_tokens, int top_k,
+                    int64_t hidden, int64_t n_out_rows, int dtype, stm_stream_t stream);
+
+/* MoEWeightedGather.forward, moe_utils.py:249-284:
+ * out[t,:] = sum_k w[t,k] * in[pos[t,k], :]; accumulation in fp32 when the weights are
+ * fp32, otherwise each product is rounded to the row dtype first (moe_utils.py:274-279). */
+int stm_unpermute_fwd(const void* in, const void* pos, int pos_is_i64, const void* weight, int weight_dtype,
+                      void* out, int64_t n_tokens, int top_k, int64_t hidden, int64_t n_in_rows, int dtype,
+                      stm_stream_t stream);
+
+/* MoEWeightedGather.backward, moe_utils.py:286-307, for an INJECTIVE pos (every row named
+ * by at most one slot -- always true for stm_index_compute output):
+ * grad_in[pos[t,k], :] = go[t,:] * w[t,k];  grad_w[t,k] = <go[t,:], in[pos[t,k], :]>.
+ * Rows of grad_in that no slot names are left untouched (see stm_zero_unwritten_rows). */
+int stm_unpermute_bwd(const void* grad_out, const void* in, const void* pos, int pos_is_i64, const void* weight,
+                      int weight_dtype, void* grad_in, void* grad_weight, int64_t n_tokens, int top_k,
+                      int64_t hidden, int64_t n_in_rows, int dtype, uint8_t* written_or_null, stm_stream_t stream);
+
+/* Inspects a position map: status[STM_ST_N_VALID] = number of non-negative entries,
+ * status[STM_ST_MAX_ROW_PLUS1] = 1 + largest entry, status[STM_ST_NOT_INJECTIVE] set when
+ * two non-negative entries are equal, status[STM_ST_ROW_OUT_OF_RANGE] when one is
+ * >= n_rows; owner: int32 [n_rows] scratch.  Serves the data-dependent sizing and checks
+ * of MoEScatter.forward (moe_utils.py:353-366) and MoEWeightedGather.backward (:302-305). */
+int stm_index_check(const void* pos, int pos_is_i64, int64_t n_slots, int64_t n_rows, int32_t* owner,
+                    int32_t* status, stm_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* STEPTRON_MOE_H_ */

@@ -1,0 +1,134 @@
+"""ctypes binding of ``libsteptron_moe_gfx950.so`` (the C ABI in ``include/steptron_moe.h``).
+
+The library is loaded from ``steptronoss_amd/lib/``; when it is missing this module
+raises -- there is no fallback implementation.  PyTorch is used for device memory and
+the current HIP stream only: every call passes raw ``data_ptr()`` values and the
+stream handle.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
+from pathlib import Path
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libsteptron_moe_gfx950.so"
+
+STM_F32, STM_F16, STM_BF16 = 0, 1, 2
+(
+    ST_ID_OUT_OF_RANGE,
+    ST_N_VALID,
+    ST_HIST_MISMATCH,
+    ST_HIST_NEGATIVE,
+    ST_NOT_INJECTIVE,
+    ST_ROW_OUT_OF_RANGE,
+    ST_MAX_ROW_PLUS1,
+) = range(7)
+STATUS_WORDS = 8
+
+_DTYPE_CODE = {torch.float32: STM_F32, torch.float16: STM_F16, torch.bfloat16: STM_BF16}
+
+P, I, L, Z, F = c_void_p, c_int, c_int64, c_size_t, c_float
+
+# name -> (restype, argtypes); must list every symbol declared in include/steptron_moe.h
+SIGNATURES = {
+    "stm_abi_version": (I, []),
+    "stm_status_string": (c_char_p, [I]),
+    "stm_route_workspace_bytes": (Z, [L, I]),
+    "stm_histogram": (I, [P, I, L, I, P, P, P, Z, P]),
+    "stm_index_compute": (I, [P, I, L, I, P, I, P, P, P, Z, P]),
+    "stm_route_plan": (I, [P, I, L, I, P, P, P, P, P, Z, P]),
+    "stm_group_offsets": (I, [P, I, I, P, P]),
+    "stm_permute_fwd": (I, [P, P, I, P, L, I, L, L, P, P]),
+    "stm_zero_unwritten_rows": (I, [P, P, L, L, P]),
+    "stm_permute_bwd": (I, [P, P, I, P, L, I, L, L, I, P]),
+    "stm_unpermute_fwd": (I, [P, P, I, P, I, P, L, I, L, L, I, P]),
+    "stm_unpermute_bwd": (I, [P, P, P, I, P, I, P, P, L, I, L, L, I, P, P]),
+    "stm_index_check": (I, [P, I, L, L, P, P, P]),
+}
+
+_lib = None
+
+
+class BackendUnavailable(RuntimeError):
+    """The HIP library is not built / not loadable, or no GPU is visible."""
+
+
+def library_path() -> Path:
+    return LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once and attach the prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise BackendUnavailable(
+            f"{LIB_PATH} is missing: build it with `python -m steptronoss_amd.build` "
+            "(the hip_gfx950 backend has no fallback implementation)"
+        )
+    try:
+        lib = ctypes.CDLL(str(LIB_PATH))
+    except OSError as exc:  # pragma: no cover - depends on the machine
+        raise BackendUnavailable(f"cannot load {LIB_PATH}: {exc}") from exc
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def status_string(code: int) -> str:
+    return load().stm_status_string(code).decode()
+
+
+def call(name: str, *args) -> None:
+    """Invoke an ``int``-returning entry point; a non-zero status raises."""
+    code = getattr(load(), name)(*args)
+    if code != 0:
+        raise RuntimeError(f"{name} failed: {status_string(code)} (status {code})")
+
+
+def ptr(t: torch.Tensor | None):
+    """Device address of a tensor's first element (``None`` -> NULL)."""
+    if t is None:
+        return None
+    return t.data_ptr() or None
+
+
+def stream() -> int:
+    """Handle of torch's current HIP stream on the current device."""
+    return torch.cuda.current_stream().cuda_stream or None
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dt]
+    except KeyError:
+        raise TypeError(f"hip_gfx950 kernels support float32/float16/bfloat16, got {dt}") from None
+
+
+def require_gpu(*tensors: torch.Tensor) -> torch.device:
+    """All tensors must be on one HIP device; returns it."""
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise BackendUnavailable(
+                "the hip_gfx950 backend only runs on GPU tensors (no CPU fallback exists); got a tensor on "
+                f"{t.device}"
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise ValueError("all tensors must be on the same device")
+    return dev
+
+
+def is_i64(t: torch.Tensor) -> int:
+    return 1 if t.dtype == torch.int64 else 0

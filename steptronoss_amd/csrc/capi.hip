@@ -1,0 +1,19 @@
+// Version / status-string entry points of the C ABI.
+#include "common.hpp"
+
+extern "C" {
+
+int stm_abi_version(void) { return 1; }
+
+const char* stm_status_string(int status) {
+  switch (status) {
+    case STM_OK: return "ok";
+    case STM_ERR_ARG: return "invalid argument (null pointer, negative size or inconsistent shapes)";
+    case STM_ERR_UNSUPPORTED: return "unsupported dtype or size";
+    case STM_ERR_WORKSPACE: return "workspace too small";
+    case STM_ERR_LAUNCH: return "HIP launch failed";
+    default: return "unknown status";
+  }
+}
+
+}  // extern "C"

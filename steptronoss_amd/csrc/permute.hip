@@ -1,0 +1,485 @@
+// Permute (token order -> expert-contiguous rows) and unpermute / weighted combine (gfx950).
+//
+// All four kernels are token-major: one workgroup owns one token, reads its row once and
+// touches the K rows its slots name.  HBM traffic is therefore exactly the compulsory
+// T*H + N*H elements (+ the index), every access is a full-row coalesced stream of 128-bit
+// words, nothing is accumulated through atomics, and the order of every sum is fixed
+// (k ascending), so results are bit-reproducible.
+#include "common.hpp"
+
+namespace stm {
+namespace {
+
+constexpr int kRowThreads = 256;
+
+template <bool I64>
+__device__ __forceinline__ int64_t load_pos(const void* pos, int64_t i) {
+  if constexpr (I64)
+    return static_cast<const int64_t*>(pos)[i];
+  else
+    return static_cast<const int32_t*>(pos)[i];
+}
+
+// ---------------------------------------------------------------- permute forward
+// Bit copy; V is the widest unit that divides the row and the base alignment.
+template <typename V, bool I64>
+__global__ __launch_bounds__(kRowThreads) void permute_fwd_kernel(const V* __restrict__ x,
+                                                                  const void* __restrict__ pos, V* __restrict__ out,
+                                                                  int top_k, int64_t units, int64_t n_out_rows,
+                                                                  uint8_t* __restrict__ written) {
+  const int64_t t = blockIdx.x;
+  const V* src = x + t * units;
+  const int64_t slot0 = t * top_k;
+  for (int64_t u = threadIdx.x; u < units; u += kRowThreads) {
+    const V v = src[u];
+    for (int k = 0; k < top_k; ++k) {
+      const int64_t p = load_pos<I64>(pos, slot0 + k);
+      if (p >= 0 && p < n_out_rows) out[p * units + u] = v;
+    }
+  }
+  if (written && threadIdx.x < top_k) {
+    for (int k = threadIdx.x; k < top_k; k += kRowThreads) {
+      const int64_t p = load_pos<I64>(pos, slot0 + k);
+      if (p >= 0 && p < n_out_rows) written[p] = 1;
+    }
+  }
+}
+
+template <typename V>
+__global__ __launch_bounds__(kRowThreads) void zero_unwritten_kernel(V* __restrict__ out,
+                                                                     const uint8_t* __restrict__ written,
+                                                                     int64_t n_rows, int64_t units) {
+  const int64_t r = int64_t(blockIdx.x) * (kRowThreads / kWave) + threadIdx.x / kWave;
+  if (r >= n_rows || written[r]) return;
+  V zero{};
+  for (int64_t u = threadIdx.x % kWave; u < units; u += kWave) out[r * units + u] = zero;
+}
+
+// ---------------------------------------------------------------- vectors of elements
+template <typename T, int VEC>
+struct alignas(sizeof(T) * VEC) Pack {
+  T v[VEC];
+};
+
+template <typename T>
+__device__ __forceinline__ float round_through(float f) {
+  return to_float(from_float<T>(f));
+}
+
+template <typename W>
+__device__ __forceinline__ float load_weight(const void* w, int64_t i) {
+  return to_float(static_cast<const W*>(w)[i]);
+}
+
+__device__ __forceinline__ float load_weight_any(const void* w, int wdtype, int64_t i) {
+  switch (wdtype) {
+    case STM_F32: return load_weight<float>(w, i);
+    case STM_F16: return load_weight<f16_t>(w, i);
+    default: return load_weight<bf16_t>(w, i);
+  }
+}
+
+__device__ __forceinline__ void store_weight_any(void* w, int wdtype, int64_t i, float f) {
+  switch (wdtype) {
+    case STM_F32: static_cast<float*>(w)[i] = f; break;
+    case STM_F16: static_cast<f16_t*>(w)[i] = from_float<f16_t>(f); break;
+    default: static_cast<bf16_t*>(w)[i] = from_float<bf16_t>(f); break;
+  }
+}
+
+// ---------------------------------------------------------------- permute backward
+// gx[t,:] = sum_k go[pos[t,k],:], fp32 accumulation, one rounding.
+template <typename T, int VEC, bool I64>
+__global__ __launch_bounds__(kRowThreads) void permute_bwd_kernel(const T* __restrict__ go,
+                                                                  const void* __restrict__ pos, T* __restrict__ gx,
+                                                                  int top_k, int64_t hidden, int64_t n_rows) {
+  using P = Pack<T, VEC>;
+  const int64_t t = blockIdx.x;
+  const int64_t units = hidden / VEC;
+  const int64_t slot0 = t * top_k;
+  for (int64_t u = threadIdx.x; u < units; u += kRowThreads) {
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+    for (int k = 0; k < top_k; ++k) {
+      const int64_t p = load_pos<I64>(pos, slot0 + k);
+      if (p < 0 || p >= n_rows) continue;
+      const P row = reinterpret_cast<const P*>(go + p * hidden)[u];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] += to_float(row.v[j]);
+    }
+    P o;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) o.v[j] = from_float<T>(acc[j]);
+    reinterpret_cast<P*>(gx + t * hidden)[u] = o;
+  }
+}
+
+// ---------------------------------------------------------------- unpermute forward
+// out[t,:] = sum_k w[t,k] * in[pos[t,k],:].  FP32W: fp32 weights => fp32 products;
+// otherwise weight and product are rounded to T before the (fp32) sum.
+template <typename T, int VEC, bool I64, bool FP32W>
+__global__ __launch_bounds__(kRowThreads) void unpermute_fwd_kernel(const T* __restrict__ in,
+                                                                    const void* __restrict__ pos,
+                                                                    const void* __restrict__ weight, int wdtype,
+                                                                    T* __restrict__ out, int top_k, int64_t hidden,
+                                                                    int64_t n_rows) {
+  using P = Pack<T, VEC>;
+  const int64_t t = blockIdx.x;
+  const int64_t units = hidden / VEC;
+  const int64_t slot0 = t * top_k;
+  for (int64_t u = threadIdx.x; u < units; u += kRowThreads) {
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+    for (int k = 0; k < top_k; ++k) {
+      const int64_t p = load_pos<I64>(pos, slot0 + k);
+      if (p < 0 || p >= n_rows) continue;
+      float w = load_weight_any(weight, wdtype, slot0 + k);
+      if constexpr (!FP32W) w = round_through<T>(w);
+      const P row = reinterpret_cast<const P*>(in + p * hidden)[u];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float prod = to_float(row.v[j]) * w;
+        acc[j] += FP32W ? prod : round_through<T>(prod);
+      }
+    }
+    P o;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) o.v[j] = from_float<T>(acc[j]);
+    reinterpret_cast<P*>(out + t * hidden)[u] = o;
+  }
+}
+
+// ---------------------------------------------------------------- unpermute backward
+// grad_in[pos[t,k],:] = go[t,:] * w[t,k] (both rounded to T), grad_w[t,k] = <go[t,:], in[pos,:]>
+// (fp32 accumulation).  Valid for an injective pos: each row is written by one slot.
+constexpr int kDotChunk = 8;
+
+template <typename T, int VEC, bool I64>
+__global__ __launch_bounds__(kRowThreads) void unpermute_bwd_kernel(
+    const T* __restrict__ go, const T* __restrict__ in, const void* __restrict__ pos, const void* __restrict__ weight,
+    int wdtype, T* __restrict__ gin, void* __restrict__ gw, int top_k, int64_t hidden, int64_t n_rows,
+    uint8_t* __restrict__ written) {
+  using P = Pack<T, VEC>;
+  __shared__ float partial[kRowThreads / kWave][kDotChunk];
+  const int64_t t = blockIdx.x;
+  const int64_t units = hidden / VEC;
+  const int64_t slot0 = t * top_k;
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  for (int k0 = 0; k0 < top_k; k0 += kDotChunk) {
+    float dot[kDotChunk];
+#pragma unroll
+    for (int c = 0; c < kDotChunk; ++c) dot[c] = 0.f;
+    for (int64_t u = threadIdx.x; u < units; u += kRowThreads) {
+      const P g = reinterpret_cast<const P*>(go + t * hidden)[u];
+#pragma unroll
+      for (int c = 0; c < kDotChunk; ++c) {
+        const int k = k0 + c;
+        if (k >= top_k) break;
+        const int64_t p = load_pos<I64>(pos, slot0 + k);
+        if (p < 0 || p >= n_rows) continue;
+        const float w = round_through<T>(load_weight_any(weight, wdtype, slot0 + k));
+        const P row = reinterpret_cast<const P*>(in + p * hidden)[u];
+        P o;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float gj = to_float(g.v[j]);
+          dot[c] += gj * to_float(row.v[j]);
+          o.v[j] = from_float<T>(gj * w);
+        }
+        reinterpret_cast<P*>(gin + p * hidden)[u] = o;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < kDotChunk; ++c) {
+      const float s = wave_sum(dot[c]);
+      if (lane == 0) partial[wave][c] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x < kDotChunk && k0 + threadIdx.x < top_k) {
+      const int k = k0 + threadIdx.x;
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < kRowThreads / kWave; ++w) s += partial[w][threadIdx.x];
+      const int64_t p = load_pos<I64>(pos, slot0 + k);
+      const bool ok = p >= 0 && p < n_rows;
+      store_weight_any(gw, wdtype, slot0 + k, ok ? s : 0.f);
+      if (ok && written) written[p] = 1;
+    }
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------- index check
+template <bool I64>
+__global__ void claim_rows_kernel(const void* __restrict__ pos, int64_t n_slots, int64_t n_rows,
+                                  int32_t* __restrict__ owner, int32_t* __restrict__ status) {
+  const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n_slots) return;
+  const int64_t p = load_pos<I64>(pos, i);
+  if (p < 0) return;
+  if (p >= n_rows) {
+    status[STM_ST_ROW_OUT_OF_RANGE] = 1;
+    return;
+  }
+  owner[p] = int32_t(i);
+}
+
+template <bool I64>
+__global__ void verify_rows_kernel(const void* __restrict__ pos, int64_t n_slots, int64_t n_rows,
+                                   const int32_t* __restrict__ owner, int32_t* __restrict__ status) {
+  const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n_slots) return;
+  const int64_t p = load_pos<I64>(pos, i);
+  if (p < 0 || p >= n_rows) return;
+  if (owner[p] != int32_t(i)) status[STM_ST_NOT_INJECTIVE] = 1;
+}
+
+// One workgroup: number of non-negative entries and 1 + the largest entry.
+template <bool I64>
+__global__ __launch_bounds__(1024) void summarize_pos_kernel(const void* __restrict__ pos, int64_t n_slots,
+                                                             int32_t* __restrict__ status) {
+  __shared__ int32_t counts[1024 / kWave];
+  __shared__ int32_t maxima[1024 / kWave];
+  int32_t n = 0, mx = 0;
+  for (int64_t i = threadIdx.x; i < n_slots; i += 1024) {
+    const int64_t p = load_pos<I64>(pos, i);
+    if (p >= 0) {
+      ++n;
+      const int32_t q = p >= INT32_MAX ? INT32_MAX : int32_t(p) + 1;
+      mx = q > mx ? q : mx;
+    }
+  }
+  n = wave_sum(n);
+  mx = wave_max(mx);
+  if (threadIdx.x % kWave == 0) {
+    counts[threadIdx.x / kWave] = n;
+    maxima[threadIdx.x / kWave] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t tn = 0, tm = 0;
+    for (int w = 0; w < 1024 / kWave; ++w) {
+      tn += counts[w];
+      tm = maxima[w] > tm ? maxima[w] : tm;
+    }
+    status[STM_ST_N_VALID] = tn;
+    status[STM_ST_MAX_ROW_PLUS1] = tm;
+  }
+}
+
+// ---------------------------------------------------------------- host dispatch
+inline int copy_unit_bytes(int64_t row_bytes, const void* a, const void* b) {
+  for (int unit : {16, 8, 4, 2}) {
+    if (row_bytes % unit == 0 && aligned_to(a, unit) && aligned_to(b, unit)) return unit;
+  }
+  return 1;
+}
+
+template <typename V>
+int launch_permute_fwd(const void* x, const void* pos, int pos_is_i64, void* out, int64_t n_tokens, int top_k,
+                       int64_t row_bytes, int64_t n_out_rows, uint8_t* written, hipStream_t s) {
+  const int64_t units = row_bytes / int64_t(sizeof(V));
+  if (pos_is_i64)
+    permute_fwd_kernel<V, true><<<unsigned(n_tokens), kRowThreads, 0, s>>>(
+        static_cast<const V*>(x), pos, static_cast<V*>(out), top_k, units, n_out_rows, written);
+  else
+    permute_fwd_kernel<V, false><<<unsigned(n_tokens), kRowThreads, 0, s>>>(
+        static_cast<const V*>(x), pos, static_cast<V*>(out), top_k, units, n_out_rows, written);
+  return launch_status();
+}
+
+template <typename T>
+constexpr int wide_vec() {
+  return 16 / int(sizeof(T));
+}
+
+template <typename T>
+bool can_vectorise(int64_t hidden, std::initializer_list<const void*> ptrs) {
+  if (hidden % wide_vec<T>() != 0) return false;
+  for (const void* p : ptrs)
+    if (!aligned_to(p, 16)) return false;
+  return true;
+}
+
+template <typename T>
+int dispatch_permute_bwd(const void* go, const void* pos, int pos_is_i64, void* gx, int64_t n_tokens, int top_k,
+                         int64_t hidden, int64_t n_rows, hipStream_t s) {
+  const T* g = static_cast<const T*>(go);
+  T* o = static_cast<T*>(gx);
+  const unsigned grid = unsigned(n_tokens);
+  const bool vec = can_vectorise<T>(hidden, {go, gx});
+#define STM_LAUNCH(VEC, I64) \
+  permute_bwd_kernel<T, VEC, I64><<<grid, kRowThreads, 0, s>>>(g, pos, o, top_k, hidden, n_rows)
+  if (vec) {
+    if (pos_is_i64) STM_LAUNCH(wide_vec<T>(), true); else STM_LAUNCH(wide_vec<T>(), false);
+  } else {
+    if (pos_is_i64) STM_LAUNCH(1, true); else STM_LAUNCH(1, false);
+  }
+#undef STM_LAUNCH
+  return launch_status();
+}
+
+template <typename T>
+int dispatch_unpermute_fwd(const void* in, const void* pos, int pos_is_i64, const void* w, int wdtype, void* out,
+                           int64_t n_tokens, int top_k, int64_t hidden, int64_t n_rows, hipStream_t s) {
+  const T* i = static_cast<const T*>(in);
+  T* o = static_cast<T*>(out);
+  const unsigned grid = unsigned(n_tokens);
+  const bool vec = can_vectorise<T>(hidden, {in, out});
+  const bool fp32w = wdtype == STM_F32;
+#define STM_LAUNCH(VEC, I64, F32W) \
+  unpermute_fwd_kernel<T, VEC, I64, F32W><<<grid, kRowThreads, 0, s>>>(i, pos, w, wdtype, o, top_k, hidden, n_rows)
+#define STM_PICK(VEC)                                                        \
+  if (pos_is_i64) {                                                          \
+    if (fp32w) STM_LAUNCH(VEC, true, true); else STM_LAUNCH(VEC, true, false);   \
+  } else {                                                                   \
+    if (fp32w) STM_LAUNCH(VEC, false, true); else STM_LAUNCH(VEC, false, false); \
+  }
+  if (vec) {
+    STM_PICK(wide_vec<T>())
+  } else {
+    STM_PICK(1)
+  }
+#undef STM_PICK
+#undef STM_LAUNCH
+  return launch_status();
+}
+
+template <typename T>
+int dispatch_unpermute_bwd(const void* go, const void* in, const void* pos, int pos_is_i64, const void* w, int wdtype,
+                           void* gin, void* gw, int64_t n_tokens, int top_k, int64_t hidden, int64_t n_rows,
+                           uint8_t* written, hipStream_t s) {
+  const T* g = static_cast<const T*>(go);
+  const T* i = static_cast<const T*>(in);
+  T* o = static_cast<T*>(gin);
+  const unsigned grid = unsigned(n_tokens);
+  const bool vec = can_vectorise<T>(hidden, {go, in, gin});
+#define STM_LAUNCH(VEC, I64)                                                                                      \
+  unpermute_bwd_kernel<T, VEC, I64><<<grid, kRowThreads, 0, s>>>(g, i, pos, w, wdtype, o, gw, top_k, hidden, n_rows, \
+                                                                 written)
+  if (vec) {
+    if (pos_is_i64) STM_LAUNCH(wide_vec<T>(), true); else STM_LAUNCH(wide_vec<T>(), false);
+  } else {
+    if (pos_is_i64) STM_LAUNCH(1, true); else STM_LAUNCH(1, false);
+  }
+#undef STM_LAUNCH
+  return launch_status();
+}
+
+inline bool bad_rows(int64_t n_tokens, int top_k, int64_t width) {
+  return n_tokens < 0 || top_k < 0 || width < 0 || n_tokens > 0x7fffffffll;
+}
+
+}  // namespace
+}  // namespace stm
+
+extern "C" {
+
+int stm_permute_fwd(const void* x, const void* pos, int pos_is_i64, void* out, int64_t n_tokens, int top_k,
+                    int64_t row_bytes, int64_t n_out_rows, uint8_t* written_or_null, stm_stream_t stream) {
+  using namespace stm;
+  if (bad_rows(n_tokens, top_k, row_bytes) || n_out_rows < 0) return STM_ERR_ARG;
+  if (n_tokens == 0 || top_k == 0 || row_bytes == 0 || n_out_rows == 0) return STM_OK;
+  if (!x || !pos || !out) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  switch (copy_unit_bytes(row_bytes, x, out)) {
+    case 16: return launch_permute_fwd<uint4>(x, pos, pos_is_i64, out, n_tokens, top_k, row_bytes, n_out_rows, written_or_null, s);
+    case 8: return launch_permute_fwd<uint2>(x, pos, pos_is_i64, out, n_tokens, top_k, row_bytes, n_out_rows, written_or_null, s);
+    case 4: return launch_permute_fwd<uint32_t>(x, pos, pos_is_i64, out, n_tokens, top_k, row_bytes, n_out_rows, written_or_null, s);
+    case 2: return launch_permute_fwd<uint16_t>(x, pos, pos_is_i64, out, n_tokens, top_k, row_bytes, n_out_rows, written_or_null, s);
+    default: return launch_permute_fwd<uint8_t>(x, pos, pos_is_i64, out, n_tokens, top_k, row_bytes, n_out_rows, written_or_null, s);
+  }
+}
+
+int stm_zero_unwritten_rows(void* out, const uint8_t* written, int64_t n_out_rows, int64_t row_bytes,
+                            stm_stream_t stream) {
+  using namespace stm;
+  if (n_out_rows < 0 || row_bytes < 0) return STM_ERR_ARG;
+  if (n_out_rows == 0 || row_bytes == 0) return STM_OK;
+  if (!out || !written) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  const int rows_per_block = kRowThreads / kWave;
+  const unsigned grid = unsigned((n_out_rows + rows_per_block - 1) / rows_per_block);
+  switch (copy_unit_bytes(row_bytes, out, out)) {
+    case 16: zero_unwritten_kernel<uint4><<<grid, kRowThreads, 0, s>>>(static_cast<uint4*>(out), written, n_out_rows, row_bytes / 16); break;
+    case 8: zero_unwritten_kernel<uint2><<<grid, kRowThreads, 0, s>>>(static_cast<uint2*>(out), written, n_out_rows, row_bytes / 8); break;
+    case 4: zero_unwritten_kernel<uint32_t><<<grid, kRowThreads, 0, s>>>(static_cast<uint32_t*>(out), written, n_out_rows, row_bytes / 4); break;
+    case 2: zero_unwritten_kernel<uint16_t><<<grid, kRowThreads, 0, s>>>(static_cast<uint16_t*>(out), written, n_out_rows, row_bytes / 2); break;
+    default: zero_unwritten_kernel<uint8_t><<<grid, kRowThreads, 0, s>>>(static_cast<uint8_t*>(out), written, n_out_rows, row_bytes); break;
+  }
+  return launch_status();
+}
+
+int stm_permute_bwd(const void* grad_out, const void* pos, int pos_is_i64, void* grad_x, int64_t n_tokens, int top_k,
+                    int64_t hidden, int64_t n_out_rows, int dtype, stm_stream_t stream) {
+  using namespace stm;
+  if (bad_rows(n_tokens, top_k, hidden) || n_out_rows < 0) return STM_ERR_ARG;
+  if (n_tokens == 0 || hidden == 0) return STM_OK;
+  if (!grad_x || (top_k > 0 && !pos) || (n_out_rows > 0 && !grad_out)) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case STM_F32: return dispatch_permute_bwd<float>(grad_out, pos, pos_is_i64, grad_x, n_tokens, top_k, hidden, n_out_rows, s);
+    case STM_F16: return dispatch_permute_bwd<f16_t>(grad_out, pos, pos_is_i64, grad_x, n_tokens, top_k, hidden, n_out_rows, s);
+    case STM_BF16: return dispatch_permute_bwd<bf16_t>(grad_out, pos, pos_is_i64, grad_x, n_tokens, top_k, hidden, n_out_rows, s);
+    default: return STM_ERR_UNSUPPORTED;
+  }
+}
+
+int stm_unpermute_fwd(const void* in, const void* pos, int pos_is_i64, const void* weight, int weight_dtype, void* out,
+                      int64_t n_tokens, int top_k, int64_t hidden, int64_t n_in_rows, int dtype,
+                      stm_stream_t stream) {
+  using namespace stm;
+  if (bad_rows(n_tokens, top_k, hidden) || n_in_rows < 0) return STM_ERR_ARG;
+  if (weight_dtype < STM_F32 || weight_dtype > STM_BF16) return STM_ERR_UNSUPPORTED;
+  if (n_tokens == 0 || hidden == 0) return STM_OK;
+  if (!out || (top_k > 0 && (!pos || !weight)) || (n_in_rows > 0 && !in)) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case STM_F32: return dispatch_unpermute_fwd<float>(in, pos, pos_is_i64, weight, weight_dtype, out, n_tokens, top_k, hidden, n_in_rows, s);
+    case STM_F16: return dispatch_unpermute_fwd<f16_t>(in, pos, pos_is_i64, weight, weight_dtype, out, n_tokens, top_k, hidden, n_in_rows, s);
+    case STM_BF16: return dispatch_unpermute_fwd<bf16_t>(in, pos, pos_is_i64, weight, weight_dtype, out, n_tokens, top_k, hidden, n_in_rows, s);
+    default: return STM_ERR_UNSUPPORTED;
+  }
+}
+
+int stm_unpermute_bwd(const void* grad_out, const void* in, const void* pos, int pos_is_i64, const void* weight,
+                      int weight_dtype, void* grad_in, void* grad_weight, int64_t n_tokens, int top_k, int64_t hidden,
+                      int64_t n_in_rows, int dtype, uint8_t* written_or_null, stm_stream_t stream) {
+  using namespace stm;
+  if (bad_rows(n_tokens, top_k, hidden) || n_in_rows < 0) return STM_ERR_ARG;
+  if (weight_dtype < STM_F32 || weight_dtype > STM_BF16) return STM_ERR_UNSUPPORTED;
+  if (n_tokens == 0 || top_k == 0) return STM_OK;
+  if (!grad_out || !pos || !weight || !grad_weight || (n_in_rows > 0 && (!in || !grad_in))) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case STM_F32: return dispatch_unpermute_bwd<float>(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k, hidden, n_in_rows, written_or_null, s);
+    case STM_F16: return dispatch_unpermute_bwd<f16_t>(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k, hidden, n_in_rows, written_or_null, s);
+    case STM_BF16: return dispatch_unpermute_bwd<bf16_t>(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k, hidden, n_in_rows, written_or_null, s);
+    default: return STM_ERR_UNSUPPORTED;
+  }
+}
+
+int stm_index_check(const void* pos, int pos_is_i64, int64_t n_slots, int64_t n_rows, int32_t* owner, int32_t* status,
+                    stm_stream_t stream) {
+  using namespace stm;
+  if (n_slots < 0 || n_rows < 0 || !status) return STM_ERR_ARG;
+  if (n_slots == 0) return STM_OK;
+  if (!pos || (n_rows > 0 && !owner)) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  const unsigned grid = unsigned((n_slots + 255) / 256);
+  if (pos_is_i64) {
+    summarize_pos_kernel<true><<<1, 1024, 0, s>>>(pos, n_slots, status);
+    claim_rows_kernel<true><<<grid, 256, 0, s>>>(pos, n_slots, n_rows, owner, status);
+    verify_rows_kernel<true><<<grid, 256, 0, s>>>(pos, n_slots, n_rows, owner, status);
+  } else {
+    summarize_pos_kernel<false><<<1, 1024, 0, s>>>(pos, n_slots, status);
+    claim_rows_kernel<false><<<grid, 256, 0, s>>>(pos, n_slots, n_rows, owner, status);
+    verify_rows_kernel<false><<<grid, 256, 0, s>>>(pos, n_slots, n_rows, owner, status);
+  }
+  return launch_status();
+}
+
+}  // extern "C"

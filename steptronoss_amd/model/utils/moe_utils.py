@@ -1,0 +1,334 @@
+"""MoE semantic ops backed by the gfx950 HIP library (backend name ``hip_gfx950``).
+
+Host-side counterpart of the reference's ``steptronoss/model/utils/moe_utils.py``: the
+same six switchable functions with the same signatures, argument checks and error
+types --
+
+    histogram, index_compute, moe_scatter, moe_weighted_gather, grouped_gemm,
+    routed_grouped_ffn
+
+-- each a thin caller of the C ABI (``include/steptron_moe.h``).  Naming follows the
+reference: ``moe_scatter`` is the *permute* (token order -> expert-contiguous rows) and
+``moe_weighted_gather`` the *unpermute / weighted combine*.
+
+There is no PyTorch implementation of the math in this package: the functions raise
+when the library is missing or a tensor is not on a GPU.  The functions are registered
+in this package's ``optimizable`` registry both as the default body and under the
+alternative name ``hip_gfx950``; ``steptronoss_amd.backend.register_backend`` adds them
+under that name to a StepTronOSS registry.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from steptronoss_amd import _lib
+from steptronoss_amd._lib import call, dtype_code, is_i64, ptr, require_gpu, stream
+from steptronoss_amd.utils.optimizable import optimizable
+
+BACKEND_NAME = "hip_gfx950"
+
+
+@dataclass
+class Settings:
+    """Run-time switches of the backend.
+
+    validate: the stand-alone ``histogram`` / ``index_compute`` read the device status
+        words back (one small host sync, as the reference's own checks do) and raise the
+        reference's errors.  ``routed_grouped_ffn`` never synchronises unless
+        ``validate_fused`` is set.
+    """
+
+    validate: bool = True
+    validate_fused: bool = False
+
+
+settings = Settings()
+
+
+def _new_status(device) -> torch.Tensor:
+    return torch.zeros(_lib.STATUS_WORDS, dtype=torch.int32, device=device)
+
+
+def _route_workspace(n_slots: int, n_experts: int, device) -> torch.Tensor:
+    nbytes = _lib.load().stm_route_workspace_bytes(n_slots, n_experts)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+# --------------------------------------------------------------------------- histogram
+def hip_histogram(top_k_rank: torch.Tensor, expert_num: int) -> torch.Tensor:
+    """Count how many slots route to each expert id (negative ids are ignored).
+
+    Drop-in for ``histogram`` (reference moe_utils.py:90-129): int32 ``[expert_num]``;
+    ``TypeError`` / ``ValueError`` as there, including "out-of-range" for an id
+    ``>= expert_num`` (checked through the device status word when
+    ``settings.validate``).
+    """
+    if not isinstance(top_k_rank, torch.Tensor):
+        raise TypeError("top_k_rank must be a torch.Tensor")
+    if top_k_rank.dtype not in (torch.int32, torch.int64):
+        raise TypeError("top_k_rank must be int32 or int64 tensor")
+    if expert_num < 0:
+        raise ValueError("expert_num must be non-negative")
+    dev = require_gpu(top_k_rank)
+    out = torch.zeros((expert_num,), device=dev, dtype=torch.int32)
+    if expert_num == 0 or top_k_rank.numel() == 0:
+        return out
+    ids = top_k_rank.contiguous()
+    n = ids.numel()
+    with torch.cuda.device(dev):
+        status = _new_status(dev)
+        ws = _route_workspace(n, expert_num, dev)
+        call("stm_histogram", ptr(ids), is_i64(ids), n, expert_num, ptr(out), ptr(status), ptr(ws), ws.numel(), stream())
+        if settings.validate and int(status[_lib.ST_ID_OUT_OF_RANGE]):
+            raise ValueError("top_k_rank contains out-of-range expert index")
+    return out
+
+
+# --------------------------------------------------------------------------- index_compute
+def hip_index_compute(indices: torch.Tensor, expert_histogram: torch.Tensor) -> torch.Tensor:
+    """Stable position of every (token, k) slot inside the expert-contiguous buffer.
+
+    Drop-in for ``index_compute`` (reference moe_utils.py:137-214): int32 ``[T, K]``,
+    negative entries copied through; data-dependent checks raise ``AssertionError`` with
+    the reference's messages when ``settings.validate``.
+    """
+    if not isinstance(indices, torch.Tensor):
+        raise TypeError("indices must be a torch.Tensor")
+    if not isinstance(expert_histogram, torch.Tensor):
+        raise TypeError("expert_histogram must be a torch.Tensor")
+    if indices.dtype not in (torch.int32, torch.int64):
+        raise TypeError("indices must be int32 or int64 tensor")
+    if expert_histogram.dtype not in (torch.int32, torch.int64):
+        raise TypeError("expert_histogram must be int32 or int64 tensor")
+    if indices.dim() != 2:
+        raise ValueError("indices must be 2D [token_num, top_k]")
+    if expert_histogram.dim() != 1:
+        raise ValueError("expert_histogram must be 1D [num_experts]")
+    if indices.device != expert_histogram.device:
+        raise ValueError("indices and expert_histogram must be on the same device")
+    dev = require_gpu(indices, expert_histogram)
+    out = torch.empty(indices.shape, device=dev, dtype=torch.int32)
+    n = indices.numel()
+    if n == 0:
+        return out
+    ids = indices.contiguous()
+    hist = expert_histogram.contiguous()
+    n_experts = hist.numel()
+    with torch.cuda.device(dev):
+        status = _new_status(dev)
+        ws = _route_workspace(n, n_experts, dev)
+        call(
+            "stm_index_compute", ptr(ids), is_i64(ids), n, n_experts, ptr(hist), is_i64(hist), ptr(out), ptr(status),
+            ptr(ws), ws.numel(), stream(),
+        )  # fmt: skip
+        if settings.validate:
+            st = status.tolist()
+            assert not st[_lib.ST_ID_OUT_OF_RANGE], "indices contains out-of-range expert index"
+            assert not st[_lib.ST_HIST_NEGATIVE], "expert_histogram must be non-negative"
+            assert not st[_lib.ST_HIST_MISMATCH], "expert_histogram does not match number of valid indices"
+    return out
+
+
+def route_plan(token_expert_ids: torch.Tensor, n_experts: int):
+    """histogram + expert row offsets + positions in one pass, no host sync.
+
+    Returns ``(hist int32 [E], offsets int32 [E+1], pos int32 [T,K], status int32[8])``.
+    """
+    dev = require_gpu(token_expert_ids)
+    ids = token_expert_ids.contiguous()
+    n = ids.numel()
+    hist = torch.empty((n_experts,), device=dev, dtype=torch.int32)
+    offsets = torch.empty((n_experts + 1,), device=dev, dtype=torch.int32)
+    pos = torch.empty(ids.shape, device=dev, dtype=torch.int32)
+    with torch.cuda.device(dev):
+        status = _new_status(dev)
+        ws = _route_workspace(n, n_experts, dev)
+        call(
+            "stm_route_plan", ptr(ids), is_i64(ids), n, n_experts, ptr(hist), ptr(offsets), ptr(pos), ptr(status),
+            ptr(ws), ws.numel(), stream(),
+        )  # fmt: skip
+    return hist, offsets, pos, status
+
+
+# --------------------------------------------------------------------------- permute
+def _check_index(index: torch.Tensor, n_rows: int):
+    """Device check of a position map; returns the status words as a python list."""
+    dev = index.device
+    status = _new_status(dev)
+    owner = torch.empty((max(n_rows, 1),), device=dev, dtype=torch.int32)
+    call("stm_index_check", ptr(index), is_i64(index), index.numel(), n_rows, ptr(owner), ptr(status), stream())
+    return status.tolist()
+
+
+def _permute_rows(x: torch.Tensor, pos: torch.Tensor, n_out_rows: int, written: torch.Tensor | None) -> torch.Tensor:
+    T, K = pos.shape
+    out = torch.empty((n_out_rows, x.shape[1]), device=x.device, dtype=x.dtype)
+    row_bytes = x.shape[1] * x.element_size()
+    call(
+        "stm_permute_fwd", ptr(x), ptr(pos), is_i64(pos), ptr(out), T, K, row_bytes, n_out_rows, ptr(written), stream()
+    )
+    return out
+
+
+def _permute_rows_bwd(grad_out: torch.Tensor, pos: torch.Tensor, hidden: int) -> torch.Tensor:
+    T, K = pos.shape
+    gx = torch.empty((T, hidden), device=grad_out.device, dtype=grad_out.dtype)
+    call(
+        "stm_permute_bwd", ptr(grad_out), ptr(pos), is_i64(pos), ptr(gx), T, K, hidden, grad_out.shape[0],
+        dtype_code(grad_out.dtype), stream(),
+    )  # fmt: skip
+    return gx
+
+
+class _MoEScatter(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+        if index.dtype not in (torch.int32, torch.int64):
+            raise TypeError("index must be int32 or int64 tensor")
+        if index.dim() != 2:
+            raise ValueError("index must be 2D [token_num, top_k]")
+        if input.dim() != 2:
+            raise ValueError("input must be 2D [token_num, hidden_dim]")
+        if input.shape[0] != index.shape[0]:
+            raise ValueError("input and index must have the same token_num")
+        dev = require_gpu(input, index)
+        x = input.contiguous()
+        pos = index.contiguous()
+        ctx.save_for_backward(pos)
+        ctx.hidden = x.shape[1]
+        if pos.numel() == 0:
+            return x.new_zeros((0, x.shape[1]))
+        with torch.cuda.device(dev):
+            # The output has one row per non-negative entry: a host-visible size, hence
+            # one read-back (the reference sizes its output the same way).
+            st = _check_index(pos, pos.numel())
+            n_out = st[_lib.ST_N_VALID]
+            if st[_lib.ST_ROW_OUT_OF_RANGE] or st[_lib.ST_MAX_ROW_PLUS1] > n_out:
+                raise IndexError("index out of range in moe_scatter")
+            bijection = not st[_lib.ST_NOT_INJECTIVE]
+            written = None if bijection else torch.zeros((max(n_out, 1),), device=dev, dtype=torch.uint8)
+            out = _permute_rows(x, pos, n_out, written)
+            if written is not None and n_out:
+                row_bytes = x.shape[1] * x.element_size()
+                call("stm_zero_unwritten_rows", ptr(out), ptr(written), n_out, row_bytes, stream())
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out: torch.Tensor):
+        (pos,) = ctx.saved_tensors
+        T = pos.shape[0]
+        if grad_out.numel() == 0 or pos.numel() == 0:
+            return grad_out.new_zeros((T, ctx.hidden)), None
+        with torch.cuda.device(grad_out.device):
+            return _permute_rows_bwd(grad_out.contiguous(), pos, ctx.hidden), None
+
+
+def hip_moe_scatter(input: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    """Permute: ``out[index[t,k], :] = input[t, :]`` for non-negative entries.
+
+    Drop-in for ``moe_scatter`` (reference moe_utils.py:337-420); differentiable in
+    ``input`` (backward = sum of the K gathered rows, fp32 accumulation).
+    """
+    return _MoEScatter.apply(input, index)
+
+
+# --------------------------------------------------------------------------- unpermute
+def _combine_rows(inp: torch.Tensor, pos: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    T, K = pos.shape
+    hidden = inp.shape[-1]
+    out = torch.empty((T, hidden), device=inp.device, dtype=inp.dtype)
+    call(
+        "stm_unpermute_fwd", ptr(inp), ptr(pos), is_i64(pos), ptr(weight), dtype_code(weight.dtype), ptr(out), T, K,
+        hidden, inp.shape[0], dtype_code(inp.dtype), stream(),
+    )  # fmt: skip
+    return out
+
+
+def _combine_rows_bwd(grad_out, inp, pos, weight, grad_in, written):
+    T, K = pos.shape
+    hidden = inp.shape[-1]
+    gw = torch.empty((T, K), device=inp.device, dtype=weight.dtype)
+    call(
+        "stm_unpermute_bwd", ptr(grad_out), ptr(inp), ptr(pos), is_i64(pos), ptr(weight), dtype_code(weight.dtype),
+        ptr(grad_in), ptr(gw), T, K, hidden, inp.shape[0], dtype_code(inp.dtype), ptr(written), stream(),
+    )  # fmt: skip
+    return gw
+
+
+class _MoEWeightedGather(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input: torch.Tensor, index: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+        if index.dtype not in (torch.int32, torch.int64):
+            raise TypeError("index must be int32 or int64 tensor")
+        if weight.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+            raise TypeError("weight must be a floating tensor")
+        if index.dim() != 2 or weight.dim() != 2:
+            raise ValueError("index and weight must be 2D [token_num, top_k]")
+        if weight.shape != index.shape:
+            raise ValueError("index and weight must have the same shape")
+        dev = require_gpu(input, index, weight)
+        inp = input.contiguous()
+        pos = index.contiguous()
+        w = weight.contiguous()
+        ctx.save_for_backward(inp, pos, w)
+        with torch.cuda.device(dev):
+            return _combine_rows(inp, pos, w)
+
+    @staticmethod
+    def backward(ctx, grad_out: torch.Tensor):
+        inp, pos, w = ctx.saved_tensors
+        dev = inp.device
+        n_rows = inp.shape[0]
+        with torch.cuda.device(dev):
+            go = grad_out.contiguous()
+            if pos.numel() == 0 or n_rows == 0:
+                return torch.zeros_like(inp), None, torch.zeros_like(w)
+            st = _check_index(pos, n_rows)
+            if st[_lib.ST_ROW_OUT_OF_RANGE]:
+                raise IndexError("index out of range in moe_weighted_gather")
+            if st[_lib.ST_NOT_INJECTIVE]:
+                raise NotImplementedError(
+                    "hip_gfx950 moe_weighted_gather backward: several slots name the same input row; "
+                    "only position maps produced by index_compute (injective) are supported"
+                )
+            grad_in = torch.empty_like(inp)
+            covers_all = st[_lib.ST_N_VALID] == n_rows
+            written = None if covers_all else torch.zeros((n_rows,), device=dev, dtype=torch.uint8)
+            gw = _combine_rows_bwd(go, inp, pos, w, grad_in, written)
+            if written is not None:
+                row_bytes = inp.shape[1] * inp.element_size()
+                call("stm_zero_unwritten_rows", ptr(grad_in), ptr(written), n_rows, row_bytes, stream())
+        return grad_in, None, gw
+
+
+def hip_moe_weighted_gather(input: torch.Tensor, index: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """Unpermute / combine: ``out[t,:] = sum_k weight[t,k] * input[index[t,k], :]``.
+
+    Drop-in for ``moe_weighted_gather`` (reference moe_utils.py:247-334); differentiable
+    in ``input`` and ``weight``.
+    """
+    return _MoEWeightedGather.apply(input, index, weight)
+
+
+# --------------------------------------------------------------------------- registry entries
+@optimizable(alternatives={BACKEND_NAME: hip_histogram})
+def histogram(top_k_rank: torch.Tensor, expert_num: int) -> torch.Tensor:
+    return hip_histogram(top_k_rank, expert_num)
+
+
+@optimizable(alternatives={BACKEND_NAME: hip_index_compute})
+def index_compute(indices: torch.Tensor, expert_histogram: torch.Tensor) -> torch.Tensor:
+    return hip_index_compute(indices, expert_histogram)
+
+
+@optimizable(alternatives={BACKEND_NAME: hip_moe_weighted_gather})
+def moe_weighted_gather(input: torch.Tensor, index: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    return hip_moe_weighted_gather(input, index, weight)
+
+
+@optimizable(alternatives={BACKEND_NAME: hip_moe_scatter})
+def moe_scatter(input: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    return hip_moe_scatter(input, index)
