@@ -202,8 +202,8 @@ def test_combine_matches_oracle(T, H, K, E, dtype, wdtype, inv):
     # oracle in the op's own dtypes (reproduces its rounding points) ...
     ref_same = O.moe_weighted_gather(rows, pos, w)
     # ... and in fp32 from the same rounded inputs
-    rr = rows.float().requires_grad_(True)
-    wr = w.float().requires_grad_(True)
+    rr = rows.clone().float().requires_grad_(True)
+    wr = w.clone().float().requires_grad_(True)
     ref32 = O.moe_weighted_gather(rr, pos, wr)
     rg = rows.to(DEV).requires_grad_(True)
     wg = w.to(DEV).requires_grad_(True)
