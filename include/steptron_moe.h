@@ -137,6 +137,28 @@ int stm_unpermute_bwd(const void* grad_out, const void* in, const void* pos, int
 int stm_index_check(const void* pos, int pos_is_i64, int64_t n_slots, int64_t n_rows, int32_t* owner,
                     int32_t* status, stm_stream_t stream);
 
+/* ------------------------------------------------------------------------------------
+ * Grouped GEMM over ragged per-expert row ranges (bf16/fp16 on the matrix cores, fp32
+ * accumulation; an any-shape fp32-FMA fallback covers fp32 and unaligned sizes).
+ * Groups are described by int32 row offsets [G+1] (see stm_group_offsets /
+ * stm_route_plan); rows >= offsets[G] are neither read nor written.
+ * ---------------------------------------------------------------------------------- */
+
+size_t stm_gemm_workspace_bytes(int64_t m_cap, int n_groups);
+
+/* grouped_gemm forward, moe_utils.py:443-453 / function_imple.py:8-22:
+ *   c[r, :] = a[r, :] @ (b_is_nk ? b[g]^T : b[g])  for rows r of group g,
+ * a:[m_cap, k], b:[G, n, k] when b_is_nk (trans_b=True) else [G, k, n], c:[m_cap, n].
+ * The same entry point serves dgrad (function_imple.py:61-68): grad_a = grad_c @ b[g]
+ * is the b_is_nk = 0 product over b viewed as [G, k'=n, n'=k], and vice versa. */
+int stm_grouped_gemm(const void* a, const void* b, void* c, const int32_t* offsets, int n_groups, int64_t m_cap, int n,
+                     int k, int b_is_nk, int dtype, void* workspace, size_t workspace_bytes, stm_stream_t stream);
+
+/* grouped_gemm wgrad, function_imple.py:54-69: out[g] = x[rows of g]^T @ y[rows of g],
+ * x:[m_cap, p], y:[m_cap, q], out:[G, p, q]; an empty group gives zeros (:56-58). */
+int stm_grouped_gemm_wgrad(const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
+                           int64_t m_cap, int p, int q, int dtype, stm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -47,6 +47,9 @@ SIGNATURES = {
     "stm_unpermute_fwd": (I, [P, P, I, P, I, P, L, I, L, L, I, P]),
     "stm_unpermute_bwd": (I, [P, P, P, I, P, I, P, P, L, I, L, L, I, P, P]),
     "stm_index_check": (I, [P, I, L, L, P, P, P]),
+    "stm_gemm_workspace_bytes": (Z, [L, I]),
+    "stm_grouped_gemm": (I, [P, P, P, P, I, L, I, I, I, I, P, Z, P]),
+    "stm_grouped_gemm_wgrad": (I, [P, P, P, P, I, L, I, I, I, P]),
 }
 
 _lib = None

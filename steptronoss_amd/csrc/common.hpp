@@ -69,6 +69,46 @@ __device__ __forceinline__ T wave_max(T v) {
   return v;
 }
 
+// In-place exclusive scan of a[0..n) in LDS by the whole workgroup; returns the total.
+// n <= 4 * blockDim.x.
+__device__ inline int32_t block_exclusive_scan(int32_t* a, int n, int32_t* wave_sums) {
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = tid / kWave;
+  const int n_waves = blockDim.x / kWave;
+  int32_t v[4];
+  int32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = tid * 4 + j;
+    v[j] = i < n ? a[i] : 0;
+    mine += v[j];
+  }
+  int32_t incl = mine;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int32_t o = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += o;
+  }
+  if (lane == kWave - 1) wave_sums[wave] = incl;
+  __syncthreads();
+  int32_t before = 0, total = 0;
+  for (int w = 0; w < n_waves; ++w) {
+    const int32_t s = wave_sums[w];
+    if (w < wave) before += s;
+    total += s;
+  }
+  int32_t run = before + incl - mine;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = tid * 4 + j;
+    if (i < n) a[i] = run;
+    run += v[j];
+  }
+  __syncthreads();
+  return total;
+}
+
 // ----- host-side helpers -------------------------------------------------------------
 inline hipStream_t as_stream(stm_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -1,0 +1,37 @@
+// Shared pieces of the grouped GEMM kernels: the ragged-M tile table and launch geometry.
+#pragma once
+#include "common.hpp"
+
+namespace stm {
+
+// One entry per M-tile of the ragged problem: which group, first row, number of rows.
+struct MTile {
+  int32_t group;
+  int32_t row0;
+  int32_t rows;
+  int32_t pad;
+};
+
+constexpr int kNumXcd = 8;  // MI355X: 8 accelerator dies, workgroups are dealt to them round-robin
+
+// Workgroup b of a launch lands on XCD b % 8.  Re-number so that consecutive logical ids
+// (which share an expert's weights / an M-tile's rows) run on the same XCD and meet in its L2.
+__device__ __forceinline__ int64_t xcd_contiguous_id(int64_t block, int64_t n_blocks_padded) {
+  const int64_t per_xcd = n_blocks_padded / kNumXcd;
+  return (block % kNumXcd) * per_xcd + block / kNumXcd;
+}
+
+inline int64_t pad_to_xcd(int64_t n_blocks) { return (n_blocks + kNumXcd - 1) / kNumXcd * kNumXcd; }
+
+// Upper bound of the number of M-tiles of height bm over G groups covering at most m_cap rows.
+inline int64_t max_m_tiles(int64_t m_cap, int n_groups, int bm) { return (m_cap + bm - 1) / bm + n_groups; }
+
+// Layout of the workspace: [0] int32 n_m_tiles (+ padding to 16 bytes), then MTile[max].
+inline size_t tile_table_bytes(int64_t m_cap, int n_groups, int bm) {
+  return 16 + size_t(max_m_tiles(m_cap, n_groups, bm)) * sizeof(MTile);
+}
+
+// Enqueue the kernel that fills the table for tiles of height bm (defined in gemm_generic.hip).
+int build_tile_table(const int32_t* offsets, int n_groups, int bm, int64_t m_cap, void* table, hipStream_t stream);
+
+}  // namespace stm

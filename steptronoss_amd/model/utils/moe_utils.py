@@ -332,3 +332,115 @@ def moe_weighted_gather(input: torch.Tensor, index: torch.Tensor, weight: torch.
 @optimizable(alternatives={BACKEND_NAME: hip_moe_scatter})
 def moe_scatter(input: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
     return hip_moe_scatter(input, index)
+
+
+# --------------------------------------------------------------------------- grouped GEMM
+def _group_offsets(batch_sizes: torch.Tensor, device) -> torch.Tensor:
+    """int32 row offsets ``[G+1]`` on ``device`` from per-group row counts."""
+    sizes = batch_sizes.to(device=device).contiguous()
+    if sizes.dtype not in (torch.int32, torch.int64):
+        sizes = sizes.to(torch.int64)
+    offsets = torch.empty((sizes.numel() + 1,), device=device, dtype=torch.int32)
+    call("stm_group_offsets", ptr(sizes), is_i64(sizes), sizes.numel(), ptr(offsets), stream())
+    return offsets
+
+
+def _gemm_workspace(m_cap: int, n_groups: int, device) -> torch.Tensor:
+    nbytes = _lib.load().stm_gemm_workspace_bytes(m_cap, n_groups)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def _gemm_rows(a: torch.Tensor, b: torch.Tensor, offsets: torch.Tensor, n: int, b_is_nk: bool, zero: bool = False):
+    """``c[r,:] = a[r,:] @ (b[g]^T if b_is_nk else b[g])`` for the rows of every group."""
+    m_cap, k = a.shape
+    n_groups = b.shape[0]
+    c = (torch.zeros if zero else torch.empty)((m_cap, n), device=a.device, dtype=a.dtype)
+    ws = _gemm_workspace(m_cap, n_groups, a.device)
+    call(
+        "stm_grouped_gemm", ptr(a), ptr(b), ptr(c), ptr(offsets), n_groups, m_cap, n, k, int(b_is_nk),
+        dtype_code(a.dtype), ptr(ws), ws.numel(), stream(),
+    )  # fmt: skip
+    return c
+
+
+def _gemm_wgrad(x: torch.Tensor, y: torch.Tensor, offsets: torch.Tensor, n_groups: int) -> torch.Tensor:
+    """``out[g] = x[rows of g]^T @ y[rows of g]`` -> ``[G, P, Q]``."""
+    m_cap, p = x.shape
+    q = y.shape[1]
+    out = torch.empty((n_groups, p, q), device=x.device, dtype=x.dtype)
+    call(
+        "stm_grouped_gemm_wgrad", ptr(x), ptr(y), ptr(out), ptr(offsets), n_groups, m_cap, p, q, dtype_code(x.dtype),
+        stream(),
+    )  # fmt: skip
+    return out
+
+
+class _GroupedGemm(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, a, b, offsets, total, trans_b):
+        n = b.shape[1] if trans_b else b.shape[2]
+        with torch.cuda.device(a.device):
+            c = _gemm_rows(a, b, offsets, n, trans_b)
+        ctx.save_for_backward(a, b, offsets)
+        ctx.trans_b = trans_b
+        ctx.total = total
+        return c if total == a.shape[0] else c[:total]
+
+    @staticmethod
+    def backward(ctx, grad_c):
+        a, b, offsets = ctx.saved_tensors
+        trans_b = ctx.trans_b
+        m_cap, k = a.shape
+        n_groups = b.shape[0]
+        grad_a = grad_b = None
+        with torch.cuda.device(a.device):
+            g = grad_c.contiguous()
+            if ctx.total != m_cap:  # rows past the last group carry no gradient
+                full = g.new_zeros((m_cap, g.shape[1]))
+                full[: ctx.total] = g
+                g = full
+            if ctx.needs_input_grad[0]:
+                # dgrad (reference function_imple.py:61-68): contraction over the output
+                # features; b is read in place, as [G, n, k] (trans_b) it is the "KN" operand
+                grad_a = _gemm_rows(g, b, offsets, k, not trans_b, zero=ctx.total != m_cap)
+            if ctx.needs_input_grad[1]:
+                # wgrad: zero for an empty group (reference function_imple.py:56-58)
+                grad_b = _gemm_wgrad(g, a, offsets, n_groups) if trans_b else _gemm_wgrad(a, g, offsets, n_groups)
+        return grad_a, grad_b, None, None, None
+
+
+def hip_grouped_gemm(mat_a_flat, mat_b, batch_sizes, trans_b=False):
+    """Per-group ``a[rows of g] @ (b[g]^T if trans_b else b[g])``, concatenated.
+
+    Drop-in for ``grouped_gemm`` (reference moe_utils.py:443-453; backward as in
+    optimizations/grouped_gemm/function_imple.py:24-69).  ``batch_sizes`` may live on the
+    host or the device; the row count of the result is its sum, which costs one small
+    read-back when it lives on the device (the reference calls ``.tolist()`` there).
+    """
+    if mat_a_flat.dim() != 2 or mat_b.dim() != 3:
+        raise ValueError("mat_a_flat must be 2D [rows, k] and mat_b 3D [groups, ., .]")
+    if mat_a_flat.dtype != mat_b.dtype:
+        raise TypeError("mat_a_flat and mat_b must have the same dtype")
+    dev = require_gpu(mat_a_flat, mat_b)
+    k = mat_a_flat.shape[1]
+    k_b = mat_b.shape[2] if trans_b else mat_b.shape[1]
+    if k != k_b:
+        raise ValueError("inner dimensions of mat_a_flat and mat_b do not match")
+    if batch_sizes.numel() != mat_b.shape[0]:
+        raise ValueError("batch_sizes must have one entry per group of mat_b")
+    a = mat_a_flat.contiguous()
+    b = mat_b.contiguous()
+    with torch.cuda.device(dev):
+        offsets = _group_offsets(batch_sizes, dev)
+        if batch_sizes.is_cuda:
+            total = int(offsets[-1])
+        else:
+            total = int(batch_sizes.sum())
+    if total > a.shape[0]:
+        raise ValueError("batch_sizes sum exceeds the number of rows of mat_a_flat")
+    return _GroupedGemm.apply(a, b, offsets, total, bool(trans_b))
+
+
+@optimizable(alternatives={BACKEND_NAME: hip_grouped_gemm})
+def grouped_gemm(mat_a_flat, mat_b, batch_sizes, trans_b=False):
+    return hip_grouped_gemm(mat_a_flat, mat_b, batch_sizes, trans_b)

@@ -1,0 +1,100 @@
+"""Grouped GEMM forward / dgrad / wgrad on the GPU against the fp32 oracle.
+
+Tolerance: rel-L2 <= 1e-2 for bf16/fp16 (inputs identical, products accumulated in fp32,
+one rounding of the output), <= 1e-5 for fp32."""
+
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from steptronoss_amd.model.utils import moe_utils as M
+from steptronoss_amd.utils.optimizable import set_optimization
+from tests.helpers import rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(autouse=True)
+def _select_backend():
+    set_optimization(default=M.BACKEND_NAME)
+    yield
+    set_optimization()
+
+
+def _run_case(sizes, k, n, trans_b, dtype, sizes_on_device, tol, seed=0):
+    gen = torch.Generator().manual_seed(seed)
+    sizes = torch.tensor(sizes, dtype=torch.int64)
+    G, Mrows = sizes.numel(), int(sizes.sum())
+    a = torch.randn(Mrows, k, generator=gen).to(dtype)
+    b = (torch.randn(G, n, k, generator=gen) if trans_b else torch.randn(G, k, n, generator=gen)).to(dtype)
+    go = torch.randn(Mrows, n, generator=gen).to(dtype)
+    ar = a.clone().float().requires_grad_(True)
+    br = b.clone().float().requires_grad_(True)
+    ref = O.grouped_gemm(ar, br, sizes, trans_b)
+    ref.backward(go.float())
+    ag = a.to(DEV).requires_grad_(True)
+    bg = b.to(DEV).requires_grad_(True)
+    out = M.grouped_gemm(ag, bg, sizes.to(DEV) if sizes_on_device else sizes, trans_b=trans_b)
+    assert out.shape == ref.shape and out.dtype == dtype
+    out.backward(go.to(DEV))
+    assert rel_l2(out, ref) <= tol, ("fwd", rel_l2(out, ref))
+    assert rel_l2(ag.grad, ar.grad) <= tol, ("dgrad", rel_l2(ag.grad, ar.grad))
+    assert rel_l2(bg.grad, br.grad) <= tol, ("wgrad", rel_l2(bg.grad, br.grad))
+    for g, m in enumerate(sizes.tolist()):
+        if m == 0:
+            assert float(bg.grad[g].abs().max()) == 0.0  # empty group => zero weight gradient
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_reference_case_tiny_unaligned(trans_b):
+    # the reference's own test shape (tests/test_grouped_gemm.py:24-49): rows of 12 bytes
+    _run_case([3, 1, 4], 8, 6, trans_b, torch.bfloat16, False, 1e-2)
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize(
+    "sizes,k,n,dtype,tol",
+    [
+        ([3, 1, 4], 8, 6, torch.float32, 1e-5),
+        ([5, 0, 70, 1], 24, 40, torch.float32, 1e-5),
+        ([64, 64], 64, 64, torch.bfloat16, 1e-2),
+        ([100, 0, 37, 1, 300], 64, 96, torch.bfloat16, 1e-2),
+        ([130, 250, 0, 0, 129, 3], 200, 264, torch.bfloat16, 1e-2),  # k not a multiple of 64
+        ([77, 200], 72, 136, torch.float16, 1e-2),
+        ([300, 20, 500], 520, 512, torch.bfloat16, 1e-2),
+    ],
+)
+def test_matches_oracle(sizes, k, n, dtype, tol, trans_b):
+    _run_case(sizes, k, n, trans_b, dtype, False, tol)
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_big_tile_path_ragged(trans_b):
+    # >= 8192 rows and n >= 512 selects the 256x256 tile; ragged sizes incl. empty and huge groups
+    sizes = [1024, 0, 3000, 17, 255, 257, 2048, 1, 0, 1600]
+    _run_case(sizes, 256, 768, trans_b, torch.bfloat16, True, 1e-2)
+
+
+def test_batch_sizes_shorter_than_rows():
+    gen = torch.Generator().manual_seed(3)
+    a = torch.randn(10, 16, generator=gen)
+    b = torch.randn(2, 8, 16, generator=gen)
+    sizes = torch.tensor([3, 4])
+    out = M.grouped_gemm(a.to(DEV), b.to(DEV), sizes, trans_b=True)
+    assert out.shape == (7, 8)
+    assert rel_l2(out, O.grouped_gemm(a, b, sizes, True)) < 1e-5
+
+
+def test_empty():
+    a = torch.zeros(0, 16, device=DEV)
+    b = torch.randn(3, 8, 16, device=DEV)
+    assert M.grouped_gemm(a, b, torch.zeros(3, dtype=torch.int64), trans_b=True).shape == (0, 8)
+
+
+def test_argument_errors():
+    a = torch.zeros(4, 16, device=DEV)
+    with pytest.raises(ValueError):
+        M.grouped_gemm(a, torch.zeros(2, 8, 12, device=DEV), torch.tensor([2, 2]), trans_b=True)
+    with pytest.raises(TypeError):
+        M.grouped_gemm(a, torch.zeros(2, 8, 16, device=DEV, dtype=torch.bfloat16), torch.tensor([2, 2]), trans_b=True)
