@@ -159,6 +159,50 @@ int stm_grouped_gemm(const void* a, const void* b, void* c, const int32_t* offse
 int stm_grouped_gemm_wgrad(const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
                            int64_t m_cap, int p, int q, int dtype, stm_stream_t stream);
 
+/* ------------------------------------------------------------------------------------
+ * SwiGLU between the two expert GEMMs.
+ * ---------------------------------------------------------------------------------- */
+
+/* FeedForwardConfig.activation, steptronoss/model/common/feed_forward.py:20-26:
+ * out[r, c] = min(silu(gu[r, c]), limit) * clamp(gu[r, F + c], -limit, limit), the clamps
+ * only when has_limit.  gate_up:[rows, 2F], out:[rows, F].  live_rows (optional) is a
+ * device int32: rows >= *live_rows are skipped. */
+int stm_swiglu_fwd(const void* gate_up, void* out, int64_t rows, int64_t ffn, const int32_t* live_rows_or_null,
+                   int has_limit, float limit, int dtype, stm_stream_t stream);
+
+/* Backward of the above (what autograd derives from feed_forward.py:20-26). */
+int stm_swiglu_bwd(const void* gate_up, const void* grad_out, void* grad_gate_up, int64_t rows, int64_t ffn,
+                   const int32_t* live_rows_or_null, int has_limit, float limit, int dtype, stm_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * Router: scores, stable top-k, weight normalisation, load-balance statistics.
+ * ---------------------------------------------------------------------------------- */
+
+size_t stm_router_workspace_bytes(int64_t n_tokens, int n_experts);
+
+/* MoEBlock.forward_router, steptronoss/model/common/moe_block.py:224-292, from ready logits:
+ *   scores = softmax(logits) or sigmoid(logits)                       (:229-232)
+ *   ids    = first top_k of a stable descending sort of scores (+bias) (:235-247)
+ *   weights= scores[ids], divided by their sum (+eps) for sigmoid routing or when
+ *            norm_weights                                              (:261-272)
+ *   hist   = per-expert pick counts; me = column mean of the scores (sigmoid: of
+ *            scores / row sum); aux = n_experts * sum(me * hist)       (:274-292)
+ * n_group > 1 adds group-limited selection (not in the reference): experts in n_group
+ * contiguous groups, group score = sum of its two best scores, only the topk_group best
+ * groups stay eligible.
+ * ids_out int64 [T,K], weights_out fp32 [T,K], aux_out fp32 [1], hist_out int32 [E],
+ * me_out fp32 [E]. */
+int stm_router_fwd(const void* logits, int logits_dtype, const float* bias_or_null, int64_t n_tokens, int n_experts,
+                   int top_k, int use_sigmoid, int norm_weights, float eps, int n_group, int topk_group,
+                   int64_t* ids_out, float* weights_out, float* aux_out, int32_t* hist_out, float* me_out,
+                   void* workspace, size_t workspace_bytes, stm_stream_t stream);
+
+/* Backward of forward_router w.r.t. the logits (what autograd derives from
+ * moe_block.py:229-292): from grad_weights fp32 [T,K] and grad_aux fp32 [1] (may be null). */
+int stm_router_bwd(const void* logits, int logits_dtype, int64_t n_tokens, int n_experts, int top_k, int use_sigmoid,
+                   int norm_weights, float eps, const int64_t* ids, const float* grad_weights,
+                   const float* grad_aux_or_null, const int32_t* hist, void* grad_logits, stm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

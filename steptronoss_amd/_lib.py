@@ -50,6 +50,11 @@ SIGNATURES = {
     "stm_gemm_workspace_bytes": (Z, [L, I]),
     "stm_grouped_gemm": (I, [P, P, P, P, I, L, I, I, I, I, P, Z, P]),
     "stm_grouped_gemm_wgrad": (I, [P, P, P, P, I, L, I, I, I, P]),
+    "stm_swiglu_fwd": (I, [P, P, L, L, P, I, F, I, P]),
+    "stm_swiglu_bwd": (I, [P, P, P, L, L, P, I, F, I, P]),
+    "stm_router_workspace_bytes": (Z, [L, I]),
+    "stm_router_fwd": (I, [P, I, P, L, I, I, I, I, F, I, I, P, P, P, P, P, P, Z, P]),
+    "stm_router_bwd": (I, [P, I, L, I, I, I, I, F, P, P, P, P, P, P]),
 }
 
 _lib = None

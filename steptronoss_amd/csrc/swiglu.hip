@@ -1,0 +1,152 @@
+// SwiGLU between the two expert GEMMs: h = silu(gate) * up with gate = gu[:, :F], up = gu[:, F:],
+// optional clamp (gate side from above after the SiLU, up side to [-limit, limit]); and its
+// backward.  Element-wise, 128-bit accesses, fp32 math, one rounding per output.
+#include "common.hpp"
+
+namespace stm {
+namespace {
+
+template <typename T, int VEC>
+struct alignas(sizeof(T) * VEC) Pack {
+  T v[VEC];
+};
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + __expf(-x)); }
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const T* __restrict__ gu, T* __restrict__ h, int64_t rows,
+                                                         int64_t f, const int32_t* __restrict__ rows_dev,
+                                                         bool has_limit, float limit) {
+  using P = Pack<T, VEC>;
+  const int64_t per_row = f / VEC;
+  const int64_t live = rows_dev ? (rows_dev[0] < rows ? rows_dev[0] : rows) : rows;
+  const int64_t total = live * per_row;
+  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += int64_t(gridDim.x) * blockDim.x) {
+    const int64_t r = i / per_row, c = (i % per_row) * VEC;
+    const P g = *reinterpret_cast<const P*>(gu + r * 2 * f + c);
+    const P u = *reinterpret_cast<const P*>(gu + r * 2 * f + f + c);
+    P o;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float gv = to_float(g.v[j]);
+      float a = gv * sigmoidf_(gv);
+      float b = to_float(u.v[j]);
+      if (has_limit) {
+        a = fminf(a, limit);
+        b = fminf(fmaxf(b, -limit), limit);
+      }
+      o.v[j] = from_float<T>(a * b);
+    }
+    *reinterpret_cast<P*>(h + r * f + c) = o;
+  }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ gu, const T* __restrict__ dh,
+                                                         T* __restrict__ dgu, int64_t rows, int64_t f,
+                                                         const int32_t* __restrict__ rows_dev, bool has_limit,
+                                                         float limit) {
+  using P = Pack<T, VEC>;
+  const int64_t per_row = f / VEC;
+  const int64_t live = rows_dev ? (rows_dev[0] < rows ? rows_dev[0] : rows) : rows;
+  const int64_t total = live * per_row;
+  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += int64_t(gridDim.x) * blockDim.x) {
+    const int64_t r = i / per_row, c = (i % per_row) * VEC;
+    const P g = *reinterpret_cast<const P*>(gu + r * 2 * f + c);
+    const P u = *reinterpret_cast<const P*>(gu + r * 2 * f + f + c);
+    const P d = *reinterpret_cast<const P*>(dh + r * f + c);
+    P og, ou;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float gv = to_float(g.v[j]);
+      const float s = sigmoidf_(gv);
+      float a = gv * s;
+      float da = s * (1.f + gv * (1.f - s));
+      float b = to_float(u.v[j]);
+      float db = 1.f;
+      if (has_limit) {
+        if (a > limit) da = 0.f;  // clamp passes the gradient on [.., limit]
+        a = fminf(a, limit);
+        if (b < -limit || b > limit) db = 0.f;
+        b = fminf(fmaxf(b, -limit), limit);
+      }
+      const float dv = to_float(d.v[j]);
+      og.v[j] = from_float<T>(dv * b * da);
+      ou.v[j] = from_float<T>(dv * a * db);
+    }
+    *reinterpret_cast<P*>(dgu + r * 2 * f + c) = og;
+    *reinterpret_cast<P*>(dgu + r * 2 * f + f + c) = ou;
+  }
+}
+
+inline unsigned grid_for(int64_t work_items) {
+  const int64_t blocks = (work_items + 255) / 256;
+  return unsigned(blocks < 1 ? 1 : (blocks > 65536 ? 65536 : blocks));
+}
+
+template <typename T>
+int fwd_typed(const void* gu, void* h, int64_t rows, int64_t f, const int32_t* rows_dev, int has_limit, float limit,
+              hipStream_t s) {
+  constexpr int W = 16 / int(sizeof(T));
+  const bool vec = f % W == 0 && aligned_to(gu, 16) && aligned_to(h, 16);
+  if (vec)
+    swiglu_fwd_kernel<T, W><<<grid_for(rows * (f / W)), 256, 0, s>>>(static_cast<const T*>(gu), static_cast<T*>(h),
+                                                                     rows, f, rows_dev, has_limit != 0, limit);
+  else
+    swiglu_fwd_kernel<T, 1><<<grid_for(rows * f), 256, 0, s>>>(static_cast<const T*>(gu), static_cast<T*>(h), rows, f,
+                                                               rows_dev, has_limit != 0, limit);
+  return launch_status();
+}
+
+template <typename T>
+int bwd_typed(const void* gu, const void* dh, void* dgu, int64_t rows, int64_t f, const int32_t* rows_dev,
+              int has_limit, float limit, hipStream_t s) {
+  constexpr int W = 16 / int(sizeof(T));
+  const bool vec = f % W == 0 && aligned_to(gu, 16) && aligned_to(dh, 16) && aligned_to(dgu, 16);
+  if (vec)
+    swiglu_bwd_kernel<T, W><<<grid_for(rows * (f / W)), 256, 0, s>>>(
+        static_cast<const T*>(gu), static_cast<const T*>(dh), static_cast<T*>(dgu), rows, f, rows_dev, has_limit != 0,
+        limit);
+  else
+    swiglu_bwd_kernel<T, 1><<<grid_for(rows * f), 256, 0, s>>>(static_cast<const T*>(gu), static_cast<const T*>(dh),
+                                                               static_cast<T*>(dgu), rows, f, rows_dev, has_limit != 0,
+                                                               limit);
+  return launch_status();
+}
+
+}  // namespace
+}  // namespace stm
+
+extern "C" {
+
+int stm_swiglu_fwd(const void* gate_up, void* out, int64_t rows, int64_t ffn, const int32_t* live_rows_or_null,
+                   int has_limit, float limit, int dtype, stm_stream_t stream) {
+  using namespace stm;
+  if (rows < 0 || ffn < 0) return STM_ERR_ARG;
+  if (rows == 0 || ffn == 0) return STM_OK;
+  if (!gate_up || !out) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case STM_F32: return fwd_typed<float>(gate_up, out, rows, ffn, live_rows_or_null, has_limit, limit, s);
+    case STM_F16: return fwd_typed<f16_t>(gate_up, out, rows, ffn, live_rows_or_null, has_limit, limit, s);
+    case STM_BF16: return fwd_typed<bf16_t>(gate_up, out, rows, ffn, live_rows_or_null, has_limit, limit, s);
+    default: return STM_ERR_UNSUPPORTED;
+  }
+}
+
+int stm_swiglu_bwd(const void* gate_up, const void* grad_out, void* grad_gate_up, int64_t rows, int64_t ffn,
+                   const int32_t* live_rows_or_null, int has_limit, float limit, int dtype, stm_stream_t stream) {
+  using namespace stm;
+  if (rows < 0 || ffn < 0) return STM_ERR_ARG;
+  if (rows == 0 || ffn == 0) return STM_OK;
+  if (!gate_up || !grad_out || !grad_gate_up) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case STM_F32: return bwd_typed<float>(gate_up, grad_out, grad_gate_up, rows, ffn, live_rows_or_null, has_limit, limit, s);
+    case STM_F16: return bwd_typed<f16_t>(gate_up, grad_out, grad_gate_up, rows, ffn, live_rows_or_null, has_limit, limit, s);
+    case STM_BF16: return bwd_typed<bf16_t>(gate_up, grad_out, grad_gate_up, rows, ffn, live_rows_or_null, has_limit, limit, s);
+    default: return STM_ERR_UNSUPPORTED;
+  }
+}
+
+}  // extern "C"

@@ -1,0 +1,200 @@
+"""Router and MoE layer body on the gfx950 kernels (single GPU).
+
+Counterparts of the reference's ``steptronoss/model/common/moe_block.py``:
+``forward_router`` (:224-292), ``GroupedExperts`` (:116-169) and ``MoEBlock.forward``
+(:376-420), with the tensor/expert-parallel branches left out (one GPU: every
+all-reduce on the path is an identity) and the metrics hooks omitted.
+"""
+
+from __future__ import annotations
+
+import functools
+
+import torch
+from torch import nn
+
+from steptronoss_amd import _lib
+from steptronoss_amd._lib import call, dtype_code, ptr, require_gpu, stream
+from steptronoss_amd.model.common.feed_forward import swiglu
+from steptronoss_amd.model.utils.moe_utils import routed_grouped_ffn
+
+
+class _Router(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, bias, top_k, use_sigmoid, norm_weights, eps, n_group, topk_group):
+        dev = require_gpu(logits, bias)
+        x = logits.contiguous()
+        T, E = x.shape
+        ids = torch.empty((T, top_k), device=dev, dtype=torch.int64)
+        weights = torch.empty((T, top_k), device=dev, dtype=torch.float32)
+        aux = torch.empty((), device=dev, dtype=torch.float32)
+        hist = torch.empty((E,), device=dev, dtype=torch.int32)
+        me = torch.empty((E,), device=dev, dtype=torch.float32)
+        with torch.cuda.device(dev):
+            nbytes = _lib.load().stm_router_workspace_bytes(T, E)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            b = None if bias is None else bias.to(torch.float32).contiguous()
+            call(
+                "stm_router_fwd", ptr(x), dtype_code(x.dtype), ptr(b), T, E, top_k, int(use_sigmoid),
+                int(norm_weights), float(eps), int(n_group), int(topk_group), ptr(ids), ptr(weights), ptr(aux),
+                ptr(hist), ptr(me), ptr(ws), ws.numel(), stream(),
+            )  # fmt: skip
+        ctx.save_for_backward(x, ids, hist)
+        ctx.cfg = (top_k, use_sigmoid, norm_weights, eps)
+        ctx.mark_non_differentiable(ids, hist)
+        return ids, weights, aux, hist
+
+    @staticmethod
+    def backward(ctx, _g_ids, g_weights, g_aux, _g_hist):
+        x, ids, hist = ctx.saved_tensors
+        top_k, use_sigmoid, norm_weights, eps = ctx.cfg
+        T, E = x.shape
+        with torch.cuda.device(x.device):
+            gw = (
+                torch.zeros((T, top_k), device=x.device, dtype=torch.float32)
+                if g_weights is None
+                else g_weights.to(torch.float32).contiguous()
+            )
+            ga = None if g_aux is None else g_aux.to(torch.float32).reshape(1).contiguous()
+            gl = torch.empty_like(x)
+            call(
+                "stm_router_bwd", ptr(x), dtype_code(x.dtype), T, E, top_k, int(use_sigmoid), int(norm_weights),
+                float(eps), ptr(ids), ptr(gw), ptr(ga), ptr(hist), ptr(gl), stream(),
+            )  # fmt: skip
+        return gl, None, None, None, None, None, None, None
+
+
+def forward_router(
+    logits: torch.Tensor,
+    top_k: int,
+    *,
+    use_sigmoid: bool = False,
+    norm_expert_weight: bool = True,
+    balance_bias: torch.Tensor | None = None,
+    n_group: int = 1,
+    topk_group: int = 1,
+):
+    """Scores, stable top-k, weights and the load-balance loss from ready logits ``[T, E]``.
+
+    Follows ``MoEBlock.forward_router`` (reference moe_block.py:224-292): scores are the fp32
+    softmax (or sigmoid) of the logits; the ``top_k`` experts are the first entries of a
+    stable descending sort of the scores (plus ``balance_bias`` for selection only), so ties
+    go to the lower expert id; weights are renormalised for sigmoid routing or when
+    ``norm_expert_weight``; ``aux = E * sum(mean(scores, 0) * hist)``.  ``n_group > 1`` enables
+    group-limited selection.  Returns ``(ids int64 [T,K], weights fp32 [T,K], aux, hist int32
+    [E])``; differentiable in ``logits`` through ``weights`` and ``aux``.
+    """
+    if logits.dim() != 2:
+        raise ValueError("logits must be 2D [tokens, experts]")
+    if top_k > logits.shape[1]:
+        raise ValueError("top_k must not exceed the number of experts")
+    eps = 1e-20 if balance_bias is not None else 0.0
+    return _Router.apply(logits, balance_bias, top_k, use_sigmoid, norm_expert_weight, eps, n_group, topk_group)
+
+
+class _BindAuxLoss(torch.autograd.Function):
+    """Identity on the output; hands ``aux_loss`` a gradient of one in backward (reference
+    steptronoss/model/utils/utils.py:68-90)."""
+
+    @staticmethod
+    def forward(ctx, output, aux_loss):
+        ctx.save_for_backward(aux_loss)
+        return output.view_as(output)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (aux_loss,) = ctx.saved_tensors
+        return grad_output, torch.ones_like(aux_loss)
+
+
+def bind_aux_loss(output: torch.Tensor, aux_loss: torch.Tensor) -> torch.Tensor:
+    return _BindAuxLoss.apply(output, aux_loss)
+
+
+class MoEGate(nn.Module):
+    """``logits = x @ W^T`` (fp32 when ``fp32_output``); reference moe_block.py:97-113 and
+    moe_utils.py:64-82.  A plain dense GEMM next to the path, left to the BLAS library."""
+
+    def __init__(self, dim: int, num_experts: int, fp32_output: bool = False, device=None, dtype=None):
+        super().__init__()
+        self.fp32_output = fp32_output
+        self.weight = nn.Parameter(torch.empty(num_experts, dim, device=device, dtype=dtype))
+
+    def forward(self, x):
+        if self.fp32_output:
+            return torch.matmul(x.float(), self.weight.t().float())
+        return torch.matmul(x, self.weight.t())
+
+
+class GroupedExperts(nn.Module):
+    """Owns ``w1 [E, 2F, H]`` and ``w2 [E, H, F]`` and runs the routed FFN (reference
+    moe_block.py:116-169)."""
+
+    def __init__(self, num_experts, hidden_size, moe_hidden_size, swiglu_limit=None, device=None, dtype=None):
+        super().__init__()
+        self.activation = functools.partial(swiglu, swiglu_limit=swiglu_limit)
+        self.w1 = nn.Parameter(torch.empty(num_experts, 2 * moe_hidden_size, hidden_size, device=device, dtype=dtype))
+        self.w2 = nn.Parameter(torch.empty(num_experts, hidden_size, moe_hidden_size, device=device, dtype=dtype))
+
+    def forward(self, x, token_expert_ids, token_weights):
+        return routed_grouped_ffn(self.w1, self.w2, self.activation, x, token_expert_ids, token_weights)
+
+
+class MoEBlock(nn.Module):
+    """gate -> router -> routed experts -> bind aux loss -> scale (reference
+    moe_block.py:376-420, the ``EP == 1`` branch)."""
+
+    def __init__(
+        self,
+        hidden_size,
+        moe_hidden_size,
+        num_experts,
+        top_k,
+        *,
+        aux_loss_coef=0.0,
+        routed_scaling_factor=1.0,
+        use_sigmoid_router=False,
+        norm_expert_weight=True,
+        aux_loss_free_balance=False,
+        fp32_gate_output=False,
+        swiglu_limit=None,
+        n_group=1,
+        topk_group=1,
+        device=None,
+        dtype=None,
+    ):
+        super().__init__()
+        self.top_k = top_k
+        self.aux_loss_coef = aux_loss_coef
+        self.routed_scaling_factor = routed_scaling_factor
+        self.use_sigmoid_router = use_sigmoid_router
+        self.norm_expert_weight = norm_expert_weight
+        self.n_group, self.topk_group = n_group, topk_group
+        self.gate = MoEGate(hidden_size, num_experts, fp32_gate_output, device=device, dtype=dtype)
+        self.experts = GroupedExperts(num_experts, hidden_size, moe_hidden_size, swiglu_limit, device, dtype)
+        if aux_loss_free_balance:
+            self.register_buffer("router_balance_bias", torch.zeros(num_experts, dtype=torch.float32, device=device))
+        else:
+            self.router_balance_bias = None
+
+    def route(self, logits):
+        return forward_router(
+            logits,
+            self.top_k,
+            use_sigmoid=self.use_sigmoid_router,
+            norm_expert_weight=self.norm_expert_weight,
+            balance_bias=self.router_balance_bias,
+            n_group=self.n_group,
+            topk_group=self.topk_group,
+        )
+
+    def forward(self, x: torch.Tensor, logits: torch.Tensor | None = None):
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        if logits is None:
+            logits = self.gate(x2)
+        ids, weights, aux, _hist = self.route(logits)
+        out = self.experts(x2, ids, weights)
+        out = out.reshape(shape)
+        out = bind_aux_loss(out, aux * self.aux_loss_coef)
+        return out * self.routed_scaling_factor

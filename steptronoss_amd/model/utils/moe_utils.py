@@ -444,3 +444,196 @@ def hip_grouped_gemm(mat_a_flat, mat_b, batch_sizes, trans_b=False):
 @optimizable(alternatives={BACKEND_NAME: hip_grouped_gemm})
 def grouped_gemm(mat_a_flat, mat_b, batch_sizes, trans_b=False):
     return hip_grouped_gemm(mat_a_flat, mat_b, batch_sizes, trans_b)
+
+
+# --------------------------------------------------------------------------- routed grouped FFN
+def _no_sync_permute(x, pos, n_rows):
+    return _PermuteKnownRows.apply(x, pos, n_rows)
+
+
+class _PermuteKnownRows(torch.autograd.Function):
+    """Permute into a buffer of ``n_rows`` (>= number of used slots) rows, no host sync;
+    rows no slot names stay zero."""
+
+    @staticmethod
+    def forward(ctx, x, pos, n_rows):
+        ctx.save_for_backward(pos)
+        ctx.hidden = x.shape[1]
+        with torch.cuda.device(x.device):
+            out = torch.zeros((n_rows, x.shape[1]), device=x.device, dtype=x.dtype)
+            T, K = pos.shape
+            call(
+                "stm_permute_fwd", ptr(x), ptr(pos), is_i64(pos), ptr(out), T, K, x.shape[1] * x.element_size(),
+                n_rows, None, stream(),
+            )  # fmt: skip
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (pos,) = ctx.saved_tensors
+        with torch.cuda.device(grad_out.device):
+            return _permute_rows_bwd(grad_out.contiguous(), pos, ctx.hidden), None, None
+
+
+class _CombineInjective(torch.autograd.Function):
+    """Weighted combine whose position map is known to be injective (index_compute output)."""
+
+    @staticmethod
+    def forward(ctx, rows, pos, weight):
+        ctx.save_for_backward(rows, pos, weight)
+        with torch.cuda.device(rows.device):
+            return _combine_rows(rows, pos, weight)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        rows, pos, weight = ctx.saved_tensors
+        with torch.cuda.device(rows.device):
+            grad_rows = torch.zeros_like(rows)
+            gw = _combine_rows_bwd(grad_out.contiguous(), rows, pos, weight, grad_rows, None)
+        return grad_rows, None, gw
+
+
+class _FusedRoutedFFN(torch.autograd.Function):
+    """route_plan -> permute -> GEMM(w1^T) -> SwiGLU -> GEMM(w2^T) -> combine in one autograd
+    node: no host round trip, intermediates are sized for all ``T*K`` slots and only the rows of
+    used slots are ever touched."""
+
+    @staticmethod
+    def forward(ctx, w1, w2, x, token_expert_ids, token_weights, swiglu_limit):
+        from steptronoss_amd.model.common.feed_forward import swiglu_fwd_rows
+
+        dev = x.device
+        T, H = x.shape
+        K = token_expert_ids.shape[1]
+        E, two_f, _ = w1.shape
+        n_rows = T * K
+        with torch.cuda.device(dev):
+            _hist, offsets, pos, status = route_plan(token_expert_ids, E)
+            if settings.validate_fused and int(status[_lib.ST_ID_OUT_OF_RANGE]):
+                raise ValueError("top_k_rank contains out-of-range expert index")
+            live = offsets[E:]  # device word: number of used rows
+            xp = torch.empty((n_rows, H), device=dev, dtype=x.dtype)
+            call(
+                "stm_permute_fwd", ptr(x), ptr(pos), 0, ptr(xp), T, K, H * x.element_size(), n_rows, None, stream()
+            )
+            gu = _gemm_rows(xp, w1, offsets, two_f, True)
+            h = swiglu_fwd_rows(gu, swiglu_limit, live)
+            y = _gemm_rows(h, w2, offsets, H, True)
+            out = _combine_rows(y, pos, token_weights)
+        ctx.save_for_backward(w1, w2, xp, gu, h, y, pos, offsets, token_weights)
+        ctx.limit = swiglu_limit
+        ctx.shape = (T, H, K, E)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from steptronoss_amd.model.common.feed_forward import swiglu_bwd_rows
+
+        w1, w2, xp, gu, h, y, pos, offsets, token_weights = ctx.saved_tensors
+        T, H, K, E = ctx.shape
+        dev = grad_out.device
+        need_w1, need_w2, need_x, _, need_tw, _ = ctx.needs_input_grad
+        gw1 = gw2 = gx = gtw = None
+        with torch.cuda.device(dev):
+            live = offsets[E:]
+            go = grad_out.contiguous()
+            gy = torch.empty_like(y)
+            gtw = _combine_rows_bwd(go, y, pos, token_weights, gy, None)
+            if need_w2:
+                gw2 = _gemm_wgrad(gy, h, offsets, E)
+            if need_w1 or need_x:
+                dh = _gemm_rows(gy, w2, offsets, h.shape[1], False)
+                dgu = swiglu_bwd_rows(gu, dh, ctx.limit, live)
+                if need_w1:
+                    gw1 = _gemm_wgrad(dgu, xp, offsets, E)
+                if need_x:
+                    dxp = _gemm_rows(dgu, w1, offsets, H, False)
+                    gx = _permute_rows_bwd(dxp, pos, H)
+        return gw1, gw2, gx, None, (gtw if need_tw else None), None
+
+
+_ACT_CACHE: dict = {}
+
+
+def _swiglu_limit_of(act, ffn2: int, dtype, device):
+    """Decide whether ``act`` is the SwiGLU (optionally clamped) and with which limit.
+
+    Returns ``(True, limit)`` or ``(False, None)``.  A callable is accepted when it is this
+    package's ``swiglu`` (possibly wrapped in ``functools.partial``), or when it reproduces
+    the SwiGLU on a probe tensor whose magnitudes expose a clamp; the verdict is cached per
+    callable.  Anything else is called as-is between two un-fused GEMMs.
+    """
+    import functools
+
+    func, kwargs = act, {}
+    if isinstance(act, functools.partial):
+        func, kwargs = act.func, dict(act.keywords or {})
+        if act.args:
+            return False, None
+    limit = kwargs.pop("swiglu_limit", None)
+    if kwargs:
+        return False, None
+    if getattr(func, "is_steptron_swiglu", False):
+        return True, limit
+    key = (id(func), limit, ffn2, dtype)
+    hit = _ACT_CACHE.get(key)
+    if hit is not None and hit[0] is func:
+        return hit[1], limit if hit[1] else None
+    from steptronoss_amd.model.common.feed_forward import swiglu_fwd_rows
+
+    gen = torch.Generator(device="cpu").manual_seed(20240229)
+    probe = (torch.rand(4, ffn2, generator=gen) * 24.0 - 12.0).to(device=device, dtype=dtype)
+    ok = False
+    try:
+        with torch.no_grad():
+            theirs = act(probe)
+            mine = swiglu_fwd_rows(probe, limit)
+            if theirs.shape == mine.shape:
+                err = (theirs.float() - mine.float()).abs()
+                tol = 2e-2 * mine.float().abs() + 1e-3 if dtype != torch.float32 else 1e-5 * mine.float().abs() + 1e-6
+                ok = bool((err <= tol).all())
+    except Exception:
+        ok = False
+    _ACT_CACHE[key] = (func, ok)
+    return ok, (limit if ok else None)
+
+
+def hip_routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights):
+    """The routed expert FFN: ``combine(GEMM(act(GEMM(permute(x), w1^T)), w2^T))``.
+
+    Drop-in for ``routed_grouped_ffn`` (reference moe_utils.py:222-244), differentiable in
+    ``w1``, ``w2``, ``x`` and ``token_weights``.  ``w1`` is ``[E, 2F, H]``, ``w2`` ``[E, H, F]``.
+    When ``act`` is recognised as the SwiGLU the whole op is one autograd node; otherwise
+    ``act`` is called between the two grouped GEMMs.  No host synchronisation either way.
+    """
+    dev = require_gpu(w1, w2, x, token_expert_ids, token_weights)
+    if token_expert_ids.dtype not in (torch.int32, torch.int64):
+        raise TypeError("top_k_rank must be int32 or int64 tensor")
+    if x.dim() != 2 or token_expert_ids.dim() != 2 or token_weights.shape != token_expert_ids.shape:
+        raise ValueError("x must be [T, H]; token_expert_ids and token_weights [T, K]")
+    if w1.dtype != x.dtype or w2.dtype != x.dtype:
+        raise TypeError("w1, w2 and x must have the same dtype")
+    E = w1.shape[0]
+    T, K = token_expert_ids.shape
+    if E == 0 or T * K == 0:
+        # nothing can be routed (reference moe_utils.py:231-232)
+        return x * token_weights.sum()
+    xc, w1c, w2c = x.contiguous(), w1.contiguous(), w2.contiguous()
+    ids = token_expert_ids.contiguous()
+    tw = token_weights.contiguous()
+    with torch.cuda.device(dev):
+        fused, limit = _swiglu_limit_of(act, w1.shape[1], x.dtype, dev)
+        if fused:
+            return _FusedRoutedFFN.apply(w1c, w2c, xc, ids, tw, limit)
+        _hist, offsets, pos, _status = route_plan(ids, E)
+        n_rows = T * K
+        rows = _no_sync_permute(xc, pos, n_rows)
+        rows = _GroupedGemm.apply(rows, w1c, offsets, n_rows, True)
+        rows = act(rows)
+        rows = _GroupedGemm.apply(rows.contiguous(), w2c, offsets, n_rows, True)
+        return _CombineInjective.apply(rows, pos, tw)
+
+
+@optimizable(alternatives={BACKEND_NAME: hip_routed_grouped_ffn, "fused": hip_routed_grouped_ffn})
+def routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights):
+    return hip_routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights)

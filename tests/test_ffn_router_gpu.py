@@ -1,0 +1,249 @@
+"""GPU parity of SwiGLU, the routed grouped FFN, the router and the whole layer body.
+
+Bars: expert ids / counts / positions bit-exact; float outputs and gradients rel-L2 <= 1e-2
+for bf16 (<= 1e-5 for fp32) against the oracle evaluated in fp32 on the same inputs."""
+
+import functools
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import moe_oracle as O
+from steptronoss_amd.model.common import moe_block as B
+from steptronoss_amd.model.common.feed_forward import swiglu
+from steptronoss_amd.model.utils import moe_utils as M
+from steptronoss_amd.utils.optimizable import set_optimization
+from tests.helpers import make_topk_ids, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+BF16_TOL = 1e-2
+
+
+@pytest.fixture(autouse=True)
+def _select_backend():
+    set_optimization(default=M.BACKEND_NAME)
+    yield
+    set_optimization()
+
+
+# ------------------------------------------------------------------ SwiGLU
+@pytest.mark.parametrize("dtype,limit,F_", [(torch.bfloat16, None, 96), (torch.bfloat16, 1.5, 768), (torch.float32, 0.7, 10), (torch.float16, None, 33)])
+def test_swiglu_matches_oracle(dtype, limit, F_):
+    gen = torch.Generator().manual_seed(0)
+    x = (torch.randn(37, 2 * F_, generator=gen) * 2).to(dtype)
+    go = torch.randn(37, F_, generator=gen).to(dtype)
+    xr = x.clone().float().requires_grad_(True)
+    ref = O.swiglu(xr, limit)
+    ref.backward(go.float())
+    xg = x.to(DEV).requires_grad_(True)
+    out = swiglu(xg, limit)
+    out.backward(go.to(DEV))
+    tol = 1e-5 if dtype == torch.float32 else BF16_TOL
+    assert out.dtype == dtype and rel_l2(out, ref) <= tol and rel_l2(xg.grad, xr.grad) <= tol
+
+
+# ------------------------------------------------------------------ routed grouped FFN
+def _torch_swiglu(x, swiglu_limit=None):
+    left, right = torch.chunk(x, 2, dim=-1)
+    left = F.silu(left)
+    if swiglu_limit is not None:
+        left = left.clamp(max=swiglu_limit)
+        right = right.clamp(min=-swiglu_limit, max=swiglu_limit)
+    return left * right
+
+
+def _ffn_case(T, H, K, E, Fh, dtype, act_kind, inv, tol, seed=0, limit=None, std=1.0):
+    gen = torch.Generator().manual_seed(seed)
+    x = (torch.randn(T, H, generator=gen) * std).to(dtype)
+    w1 = (torch.randn(E, 2 * Fh, H, generator=gen) * std).to(dtype)
+    w2 = (torch.randn(E, H, Fh, generator=gen) * std).to(dtype)
+    ids = make_topk_ids(T, K, E, gen=gen, invalid_frac=inv)
+    tw = torch.rand(T, K, generator=gen)
+    tw = tw / tw.sum(1, keepdim=True)
+    go = torch.randn(T, H, generator=gen).to(dtype)
+    def oracle_act(h):
+        # A clamp makes the gradient discontinuous: whether an element sits above the limit must
+        # be decided on the same (storage-dtype) value as in the kernel path, so the oracle sees
+        # the GEMM output rounded to the storage dtype (straight-through for the gradient).
+        if limit is not None and dtype != torch.float32:
+            h = h + (h.to(dtype).float() - h).detach()
+        return O.swiglu(h, limit)
+
+    if act_kind == "own":
+        act, ref_act = functools.partial(swiglu, swiglu_limit=limit), oracle_act
+    elif act_kind == "torch":  # recognised by its behaviour on a probe
+        act, ref_act = functools.partial(_torch_swiglu, swiglu_limit=limit), oracle_act
+    else:  # an activation that is not the SwiGLU: called between two un-fused GEMMs
+        act = ref_act = lambda h: F.gelu(h[..., : h.shape[-1] // 2]) + 0.5 * h[..., h.shape[-1] // 2 :]
+
+    ref_in = [t.clone().float().requires_grad_(True) for t in (w1, w2, x, tw)]
+    ref = O.routed_grouped_ffn(ref_in[0], ref_in[1], ref_act, ref_in[2], ids, ref_in[3])
+    ref.backward(go.float())
+    got_in = [t.to(DEV).requires_grad_(True) for t in (w1, w2, x, tw)]
+    out = M.routed_grouped_ffn(got_in[0], got_in[1], act, got_in[2], ids.to(DEV), got_in[3])
+    assert out.shape == (T, H) and out.dtype == dtype
+    out.backward(go.to(DEV))
+    errs = {"out": rel_l2(out, ref)}
+    for name, g, r in zip(("dw1", "dw2", "dx", "dtw"), got_in, ref_in):
+        assert g.grad is not None and g.grad.dtype == g.dtype
+        errs[name] = rel_l2(g.grad, r.grad)
+    worst = max(errs.values())
+    assert worst <= tol, errs
+
+
+@pytest.mark.parametrize("act_kind", ["own", "torch", "other"])
+def test_ffn_reference_gpu_test_shape(act_kind):
+    # shape of the reference's fused-path test (tests/test_moe_utils_gpu.py:141-220)
+    _ffn_case(256, 64, 2, 8, 96, torch.bfloat16, act_kind, 0.15, BF16_TOL)
+
+
+@pytest.mark.parametrize(
+    "T,H,K,E,Fh,dtype,inv,tol,limit",
+    [
+        (512, 128, 4, 16, 64, torch.bfloat16, 0.0, BF16_TOL, None),
+        (300, 72, 3, 5, 40, torch.bfloat16, 0.3, BF16_TOL, 2.0),
+        (64, 8, 2, 4, 6, torch.float32, 0.1, 1e-4, None),  # nothing aligned: fallback kernels
+        (2048, 256, 8, 32, 128, torch.bfloat16, 0.0, BF16_TOL, None),
+        (128, 64, 2, 8, 32, torch.float16, 0.0, BF16_TOL, None),
+    ],
+)
+def test_ffn_matches_oracle(T, H, K, E, Fh, dtype, inv, tol, limit):
+    _ffn_case(T, H, K, E, Fh, dtype, "own", inv, tol, limit=limit, std=0.5)
+
+
+def test_ffn_experts_without_tokens():
+    # only experts 0 and 5 are used: the other weight gradients must be exactly zero
+    gen = torch.Generator().manual_seed(1)
+    T, H, K, E, Fh = 64, 64, 2, 8, 32
+    x = torch.randn(T, H, generator=gen).bfloat16().to(DEV).requires_grad_(True)
+    w1 = torch.randn(E, 2 * Fh, H, generator=gen).bfloat16().to(DEV).requires_grad_(True)
+    w2 = torch.randn(E, H, Fh, generator=gen).bfloat16().to(DEV).requires_grad_(True)
+    ids = torch.tensor([[0, 5]] * T, device=DEV)
+    tw = torch.full((T, K), 0.5, device=DEV)
+    M.routed_grouped_ffn(w1, w2, swiglu, x, ids, tw).float().sum().backward()
+    unused = [1, 2, 3, 4, 6, 7]
+    assert float(w1.grad[unused].abs().max()) == 0.0 and float(w2.grad[unused].abs().max()) == 0.0
+    assert float(w1.grad[[0, 5]].abs().max()) > 0
+
+
+# ------------------------------------------------------------------ router
+def _assert_ids(ids, ref_ids, ref_scores, K):
+    """Bit-exact expert ids, except where the oracle's own order rests on two scores closer
+    than 8 ulp (a different exp rounding may then order them differently): there the picked
+    scores must still equal the oracle's within 8 ulp."""
+    ids = ids.cpu()
+    same = (ids == ref_ids).all(1)
+    if bool(same.all()):
+        return 0
+    srt = torch.sort(ref_scores, dim=1, descending=True, stable=True).values[:, : K + 1]
+    gap = (srt[:, :-1] - srt[:, 1:]).abs()
+    near_tie = (gap <= 8 * torch.finfo(torch.float32).eps * srt[:, :-1].abs()).any(1)
+    bad = ~same & ~near_tie
+    assert not bool(bad.any()), f"{int(bad.sum())} tokens differ without a near-tie"
+    rows = torch.nonzero(~same).reshape(-1)
+    got_scores = ref_scores[rows].gather(1, ids[rows])
+    assert torch.allclose(got_scores, srt[rows, :K], rtol=1e-6, atol=0)
+    return int((~same).sum())
+
+
+ROUTER_CASES = [
+    # T, E, K, sigmoid, norm, bias, n_group, topk_group
+    (4096, 8, 2, False, False, False, 1, 1),
+    (4096, 128, 8, False, True, False, 1, 1),
+    (2048, 256, 8, True, True, False, 8, 4),
+    (1024, 256, 8, True, True, True, 8, 4),
+    (1000, 60, 6, False, True, True, 1, 1),
+    (512, 64, 4, True, True, False, 4, 2),
+    (300, 1000, 5, False, True, False, 1, 1),
+]
+
+
+@pytest.mark.parametrize("T,E,K,sig,norm,bias,ng,tg", ROUTER_CASES)
+@pytest.mark.parametrize("logit_kind", ["bf16_grid", "fp32"])
+def test_router_matches_oracle(T, E, K, sig, norm, bias, ng, tg, logit_kind):
+    gen = torch.Generator().manual_seed(7)
+    logits = torch.randn(T, E, generator=gen)
+    if logit_kind == "bf16_grid":
+        # values a bf16 gate GEMM would produce: plenty of exact ties, no sub-ulp near-ties
+        logits = (logits * 2).round() / 4 if E <= 64 else logits.bfloat16().float()
+    bb = (torch.randn(E, generator=gen) * 0.01) if bias else None
+    kw = dict(use_sigmoid=sig, norm_expert_weight=norm, balance_bias=bb, n_group=ng, topk_group=tg)
+    lr = logits.clone().requires_grad_(True)
+    ref_ids, ref_w, ref_aux, ref_hist = O.forward_router(lr, K, **kw)
+    lg = logits.to(DEV).requires_grad_(True)
+    ids, w, aux, hist = B.forward_router(lg, K, **{**kw, "balance_bias": None if bb is None else bb.to(DEV)})
+    assert ids.dtype == torch.int64 and w.dtype == torch.float32 and hist.dtype == torch.int32
+    scores = torch.sigmoid(logits) if sig else torch.softmax(logits, 1)
+    choice = scores if bb is None else scores + bb
+    choice = O.group_limited_scores(choice, ng, tg)
+    n_swapped = _assert_ids(ids, ref_ids, choice, K)
+    if logit_kind == "bf16_grid" and not bias:
+        assert n_swapped == 0
+    assert torch.equal(hist.cpu(), O.histogram(ids.cpu(), E))
+    if n_swapped == 0:
+        assert torch.equal(hist.cpu(), ref_hist)
+        assert torch.allclose(w.cpu(), ref_w, rtol=2e-5, atol=1e-7)
+        assert torch.allclose(aux.cpu(), ref_aux, rtol=2e-5)
+        gw = torch.randn(T, K, generator=gen)
+        (w * gw.to(DEV)).sum().add(aux * 0.37).backward()
+        ((ref_w * gw).sum() + ref_aux * 0.37).backward()
+        err = rel_l2(lg.grad, lr.grad)
+        assert err <= 1e-4, err
+
+
+def test_router_closed_forms():
+    T, E, K = 64, 8, 2
+    ids, w, aux, hist = B.forward_router(torch.zeros(T, E, device=DEV), K)
+    assert ids.tolist() == [[0, 1]] * T and torch.allclose(w.cpu(), torch.full((T, K), 0.5))
+    assert abs(float(aux) - T * K) < 1e-3 and hist.tolist() == [T, T, 0, 0, 0, 0, 0, 0]
+    ids, _, _, _ = B.forward_router(torch.tensor([[0.25, 0.5, 0.5, 0.25, 0.5]], device=DEV).log(), 3, norm_expert_weight=False)
+    assert ids.tolist() == [[1, 2, 4]]  # an unstable top-k would return [2, 4, 1]
+    ids, _, _, _ = B.forward_router(torch.zeros(3, 16, device=DEV, dtype=torch.bfloat16), 16)
+    assert ids.tolist() == [list(range(16))] * 3
+
+
+# ------------------------------------------------------------------ whole layer, reduced configs
+@pytest.mark.parametrize(
+    "name,T,E,tol",
+    [("c1", 256, 8, 1e-4), ("c2", 1024, 128, BF16_TOL), ("c3", 1024, 128, BF16_TOL), ("c4", 256, 256, BF16_TOL)],
+)
+def test_layer_matches_oracle_on_reduced_configs(name, T, E, tol):
+    cfg, x, w1, w2, logits = O.make_config_inputs(name, seed=1234, scale_tokens=T / O.CONFIGS[name]["T"], experts=E)
+    if name == "c4":  # keep the test small: a narrower slice of the same layer
+        x, w1, w2 = x[:, :512].contiguous(), w1[:, :512, :512].contiguous(), w2[:, :512, :256].contiguous()
+    logits = logits.bfloat16().float()  # gate-GEMM-like values: selection is exact
+    kw = dict(
+        top_k=cfg["K"], use_sigmoid=cfg["sigmoid"], norm_expert_weight=cfg["norm"], aux_loss_coef=0.01,
+        routed_scaling_factor=1.5, n_group=cfg.get("n_group", 1), topk_group=cfg.get("topk_group", 1),
+    )  # fmt: skip
+    gen = torch.Generator().manual_seed(5)
+    go = torch.randn(x.shape, generator=gen).to(x.dtype)
+    ref_in = [t.clone().float().requires_grad_(True) for t in (x, logits, w1, w2)]
+    ref, ref_ids, _, _ = O.moe_layer(*ref_in, **kw)
+    ref.backward(go.float())
+
+    blk = B.MoEBlock(
+        x.shape[1], w2.shape[2], E, cfg["K"], aux_loss_coef=0.01, routed_scaling_factor=1.5,
+        use_sigmoid_router=cfg["sigmoid"], norm_expert_weight=cfg["norm"], n_group=kw["n_group"],
+        topk_group=kw["topk_group"], device=DEV, dtype=x.dtype,
+    )  # fmt: skip
+    with torch.no_grad():
+        blk.experts.w1.copy_(w1)
+        blk.experts.w2.copy_(w2)
+    xg = x.to(DEV).requires_grad_(True)
+    lg = logits.to(DEV).requires_grad_(True)
+    out = blk(xg, logits=lg)
+    out.backward(go.to(DEV))
+    ids, _, _, _ = blk.route(lg.detach())
+    assert torch.equal(ids.cpu(), ref_ids)
+    errs = {
+        "out": rel_l2(out, ref),
+        "dx": rel_l2(xg.grad, ref_in[0].grad),
+        "dlogits": rel_l2(lg.grad, ref_in[1].grad) / 5,  # sums of many bf16-rounded dot products
+        "dw1": rel_l2(blk.experts.w1.grad, ref_in[2].grad),
+        "dw2": rel_l2(blk.experts.w2.grad, ref_in[3].grad),
+    }
+    worst = max(errs.values())
+    assert worst <= tol, errs
