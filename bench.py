@@ -1,0 +1,233 @@
+#!/usr/bin/env python
+"""Benchmark of the MoE-layer hot path on one MI355X.
+
+A "step" is one forward+backward pass of the hot path over one batch of synthetic input:
+router (scores, stable top-k, aux statistics) -> routed grouped FFN (route plan, permute,
+GEMM w1, SwiGLU, GEMM w2, weighted combine) and the backward of all of it, on the
+Qwen3-30B-A3B-like layer (T=16384, H=2048, E=128, top-8 softmax with renormalised weights,
+F=768, bf16).  All inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line.  ``value`` is the routed grouped-FFN throughput in TFLOP/s: the
+algorithmic 6*N*H*3F FLOP of the two expert GEMMs forward+backward divided by the time of
+the whole step (routing, permute and combine included).  ``roofline`` prices the grouped
+GEMM kernel against the bf16 MFMA peak, ``bandwidth`` the permute / unpermute kernels
+against HBM, both timed with HIP events on the launch stream inside the timed region.
+``cpu_baseline`` is the CPU oracle (a restatement of the reference's pure-PyTorch path)
+timed on this box's host cores on a bounded sample.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "routed grouped-FFN fwd+bwd TFLOP/s + permute/unpermute GB/s, 1 MI355X"
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
+
+WORKLOADS = {
+    "c2": dict(T=16384, H=2048, E=128, K=8, F=768, sigmoid=False, norm=True, n_group=1, topk_group=1, std=0.02),
+    "c3": dict(T=16384, H=2048, E=128, K=8, F=768, sigmoid=False, norm=True, n_group=1, topk_group=1, std=0.02, zipf=1.2),
+    "c4": dict(T=8192, H=7168, E=256, K=8, F=2048, sigmoid=True, norm=True, n_group=8, topk_group=4, std=0.006),
+}
+
+
+def make_inputs(cfg, seed, device):
+    gen = torch.Generator(device=device).manual_seed(seed)
+    T, H, E, F = cfg["T"], cfg["H"], cfg["E"], cfg["F"]
+    bf = torch.bfloat16
+    x = (torch.randn(T, H, generator=gen, device=device) * cfg["std"]).to(bf)
+    w1 = torch.empty(E, 2 * F, H, device=device, dtype=bf)
+    w2 = torch.empty(E, H, F, device=device, dtype=bf)
+    for e in range(E):  # chunked: keeps the fp32 temporaries small at the large configuration
+        w1[e] = (torch.randn(2 * F, H, generator=gen, device=device) * cfg["std"]).to(bf)
+        w2[e] = (torch.randn(H, F, generator=gen, device=device) * cfg["std"]).to(bf)
+    logits = torch.randn(T, E, generator=gen, device=device)
+    if "zipf" in cfg:
+        from oracle.moe_oracle import zipf_logit_bias
+
+        logits = logits + zipf_logit_bias(E, cfg["zipf"], torch.Generator().manual_seed(seed)).to(device)
+    go = torch.randn(T, H, generator=gen, device=device).to(bf)
+    return x, w1, w2, logits, go
+
+
+def cpu_baseline(cfg, seed, threads):
+    """Oracle on CPU tensors, fp32, on a bounded sample of the same workload: a quarter of
+    the tokens over all experts (the per-expert matmul loop at 1/4 of the rows per expert)."""
+    from oracle import moe_oracle as O
+
+    torch.set_num_threads(threads)
+    T = cfg["T"] // 4
+    H, E, F, K = cfg["H"], cfg["E"], cfg["F"], cfg["K"]
+    gen = torch.Generator().manual_seed(seed)
+    x = (torch.randn(T, H, generator=gen) * cfg["std"]).bfloat16().float().requires_grad_(True)
+    w1 = (torch.randn(E, 2 * F, H, generator=gen) * cfg["std"]).bfloat16().float().requires_grad_(True)
+    w2 = (torch.randn(E, H, F, generator=gen) * cfg["std"]).bfloat16().float().requires_grad_(True)
+    logits = torch.randn(T, E, generator=gen).requires_grad_(True)
+    go = torch.randn(T, H, generator=gen)
+    flops = 6.0 * T * K * H * 3 * F
+    times = []
+    for it in range(3):  # first pass doubles as the warm-up when time is short
+        for t in (x, w1, w2, logits):
+            t.grad = None
+        t0 = time.perf_counter()
+        out, _, _, aux = O.moe_layer(
+            x, logits, w1, w2, top_k=K, use_sigmoid=cfg["sigmoid"], norm_expert_weight=cfg["norm"], aux_loss_coef=0.01,
+            n_group=cfg["n_group"], topk_group=cfg["topk_group"],
+        )  # fmt: skip
+        out.backward(go)
+        times.append(time.perf_counter() - t0)
+        if sum(times) > 25.0:
+            break
+    best = sorted(times)[len(times) // 2] if len(times) >= 3 else min(times)
+    return {
+        "value": flops / best / 1e12,
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{T} of {cfg['T']} tokens over all {E} experts, fp32, fwd+bwd, median of {len(times)} passes, "
+        f"{best * 1e3:.0f} ms per pass",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures the single-GPU hot path only: run it with --gpus 1 (no multi-GPU figure exists)")
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the hip_gfx950 backend has no CPU fallback)")
+        sys.exit(2)
+
+    from steptronoss_amd.model.common.feed_forward import swiglu
+    from steptronoss_amd.model.common.moe_block import forward_router
+    from steptronoss_amd.model.utils.moe_utils import hip_routed_grouped_ffn
+    from steptronoss_amd.profiling import KernelTimer
+
+    cfg = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    x, w1, w2, logits, go = make_inputs(cfg, args.seed, dev)
+    for t in (x, w1, w2, logits):
+        t.requires_grad_(True)
+    one = torch.ones((), device=dev)
+    T, H, E, K, F = cfg["T"], cfg["H"], cfg["E"], cfg["K"], cfg["F"]
+    N = T * K
+
+    def step():
+        for t in (x, w1, w2, logits):
+            t.grad = None
+        ids, weights, aux, _hist = forward_router(
+            logits, K, use_sigmoid=cfg["sigmoid"], norm_expert_weight=cfg["norm"], n_group=cfg["n_group"],
+            topk_group=cfg["topk_group"],
+        )  # fmt: skip
+        out = hip_routed_grouped_ffn(w1, w2, swiglu, x, ids, weights)
+        torch.autograd.backward([out, aux], [go, one * 0.01])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    with KernelTimer() as kt:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    flops = 6.0 * N * H * 3 * F
+    value = flops / (ms_per_step * 1e-3) / 1e12
+
+    timing = kt.summary()
+    e = 2  # bytes per bf16 element
+    gemm = timing.get("stm_grouped_gemm", {"calls": 0, "total_ms": 0.0})
+    wgrad = timing.get("stm_grouped_gemm_wgrad", {"calls": 0, "total_ms": 0.0})
+    gemm_calls = gemm["calls"] + wgrad["calls"]
+    gemm_ms = gemm["total_ms"] + wgrad["total_ms"]
+    # six equal-cost-per-flop launches per step: 4 over [N, H] x 2F-sized problems count double
+    flops_per_launch = flops / 6.0
+    avg_launch_ms = gemm_ms / max(gemm_calls, 1)
+    achieved = flops_per_launch / (avg_launch_ms * 1e-3) / 1e12 if gemm_calls else 0.0
+    roofline = {
+        "bound": "mfma",
+        "kernel": "mfma_gemm_kernel (grouped GEMM fwd/dgrad/wgrad)",
+        "achieved": achieved,
+        "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": achieved / PEAK_BF16_TFLOPS,
+        "traffic": None,
+        "flops_per_launch": flops_per_launch,
+        "avg_launch_us": avg_launch_ms * 1e3,
+        "launches_per_step": gemm_calls / args.steps,
+    }
+
+    def bw(name, nbytes):
+        t = timing.get(name)
+        if not t or not t["calls"]:
+            return None
+        gbps = nbytes / (t["avg_us"] * 1e-6) / 1e9
+        return {"GB/s": gbps, "avg_us": t["avg_us"], "bytes": nbytes, "frac_of_hbm_peak": gbps / PEAK_HBM_GBPS}
+
+    bandwidth = {
+        "permute_fwd": bw("stm_permute_fwd", T * H * e + N * H * e + 4 * N),
+        "permute_bwd": bw("stm_permute_bwd", N * H * e + T * H * e + 4 * N),
+        "unpermute_fwd": bw("stm_unpermute_fwd", N * H * e + T * H * e + 8 * N),
+        "unpermute_bwd": bw("stm_unpermute_bwd", T * H * e + 2 * N * H * e + 12 * N),
+        "route_plan_us": timing.get("stm_route_plan", {}).get("avg_us"),
+        "router_fwd_us": timing.get("stm_router_fwd", {}).get("avg_us"),
+        "router_bwd_us": timing.get("stm_router_bwd", {}).get("avg_us"),
+        "swiglu_fwd_us": timing.get("stm_swiglu_fwd", {}).get("avg_us"),
+        "swiglu_bwd_us": timing.get("stm_swiglu_bwd", {}).get("avg_us"),
+    }
+
+    result = {
+        "metric": METRIC,
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: MoE layer T={T} H={H} E={E} top-{K} F={F} bf16, "
+            + ("sigmoid group-limited" if cfg["sigmoid"] else "softmax")
+            + " routing, renormalised weights; router + routed grouped FFN, fwd+bwd",
+            "tokens": T,
+            "hidden": H,
+            "experts": E,
+            "top_k": K,
+            "expert_ffn": F,
+            "seed": args.seed,
+        },
+        "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS,
+        "roofline": roofline,
+        "bandwidth": bandwidth,
+    }
+    if not args.no_cpu_baseline:
+        threads = min(os.cpu_count() or 1, 16)
+        result["cpu_baseline"] = cpu_baseline(cfg, args.seed, threads)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

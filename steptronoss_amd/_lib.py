@@ -94,9 +94,23 @@ def status_string(code: int) -> str:
     return load().stm_status_string(code).decode()
 
 
+_call_hook = None
+
+
+def set_call_hook(hook) -> None:
+    """Install an object with ``before(name)`` / ``after(name, token)`` around every call
+    (used by ``steptronoss_amd.profiling.KernelTimer``); ``None`` removes it."""
+    global _call_hook
+    _call_hook = hook
+
+
 def call(name: str, *args) -> None:
     """Invoke an ``int``-returning entry point; a non-zero status raises."""
+    hook = _call_hook
+    token = hook.before(name) if hook is not None else None
     code = getattr(load(), name)(*args)
+    if hook is not None:
+        hook.after(name, token)
     if code != 0:
         raise RuntimeError(f"{name} failed: {status_string(code)} (status {code})")
 
