@@ -31,6 +31,22 @@ inline size_t tile_table_bytes(int64_t m_cap, int n_groups, int bm) {
   return 16 + size_t(max_m_tiles(m_cap, n_groups, bm)) * sizeof(MTile);
 }
 
+// Arguments shared by the MFMA kernels (rows form: n_j = N, n_k = K; wgrad form: n_i = P, n_j = Q).
+struct GemmArgs {
+  const void* a;
+  const void* b;
+  void* c;
+  const int32_t* offsets;
+  const int32_t* header;  // rows form: header[0] = number of M-tiles in `tiles`
+  const MTile* tiles;
+  int64_t lda, ldb, ldc;
+  int64_t b_group, c_group;
+  int n_i, n_j, n_k;
+  int tiles_i, tiles_j;
+  int n_groups;
+  int64_t blocks_padded;
+};
+
 // Enqueue the kernel that fills the table for tiles of height bm (defined in gemm_generic.hip).
 int build_tile_table(const int32_t* offsets, int n_groups, int bm, int64_t m_cap, void* table, hipStream_t stream);
 

@@ -16,6 +16,11 @@
 #include "gemm_common.hpp"
 
 namespace stm {
+
+int launch_dma_rows(int dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap, int b_is_nk,
+                    void* ws, hipStream_t s);
+int launch_dma_wgrad(int dtype, const GemmArgs& base, int n_groups, int64_t m_cap, hipStream_t s);
+
 namespace {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -106,20 +111,7 @@ __device__ __forceinline__ uint4 read_fragment(const T* lds, int r0, int kk) {
   }
 }
 
-struct MfmaArgs {
-  const void* a;
-  const void* b;
-  void* c;
-  const int32_t* offsets;
-  const int32_t* header;
-  const MTile* tiles;
-  int64_t lda, ldb, ldc;
-  int64_t b_group, c_group;
-  int n_i, n_j, n_k;  // rows form: n_j = N, n_k = K;  wgrad: n_i = P, n_j = Q
-  int tiles_i, tiles_j;
-  int n_groups;
-  int64_t blocks_padded;
-};
+using MfmaArgs = GemmArgs;
 
 template <typename T>
 struct alignas(sizeof(T) * 4) Pack4 {
@@ -332,6 +324,11 @@ int launch_mfma_rows(int dtype, const void* a, const void* b, void* c, const int
   p.b_group = int64_t(n) * k;
   p.n_j = n;
   p.n_k = k;
+  p.n_groups = n_groups;
+  if (m_cap >= 4096 && n >= 256) {  // enough work for 256x256 tiles: the buffer_load->LDS kernels
+    const int st = launch_dma_rows(dtype, p, offsets, n_groups, m_cap, b_is_nk, ws, s);
+    if (st != STM_ERR_UNSUPPORTED) return st;
+  }
   return dtype == STM_BF16 ? rows_typed<bf16_t>(p, offsets, n_groups, m_cap, b_is_nk, ws, s)
                            : rows_typed<f16_t>(p, offsets, n_groups, m_cap, b_is_nk, ws, s);
 }
@@ -354,6 +351,10 @@ int launch_mfma_wgrad(int dtype, const void* x, const void* y, void* out, const 
   p.n_i = p_dim;
   p.n_j = q_dim;
   p.n_groups = n_groups;
+  if (p_dim >= 256 && q_dim >= 256) {
+    const int st = launch_dma_wgrad(dtype, p, n_groups, m_cap, s);
+    if (st != STM_ERR_UNSUPPORTED) return st;
+  }
   return dtype == STM_BF16 ? wgrad_typed<bf16_t>(p, n_groups, s) : wgrad_typed<f16_t>(p, n_groups, s);
 }
 
