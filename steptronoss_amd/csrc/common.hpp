@@ -37,7 +37,8 @@ __device__ __forceinline__ float from_float<float>(float f) {
 }
 template <>
 __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
-  return bf16_t{f32_to_bf16_bits(f)};
+  // the hardware conversion of gfx950 (v_cvt_pk_bf16_f32): round to nearest even, quiet NaNs
+  return bf16_t{__builtin_bit_cast(uint16_t, static_cast<__bf16>(f))};
 }
 template <>
 __device__ __forceinline__ f16_t from_float<f16_t>(float f) {

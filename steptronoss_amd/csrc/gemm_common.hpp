@@ -16,9 +16,15 @@ constexpr int kNumXcd = 8;  // MI355X: 8 accelerator dies, workgroups are dealt 
 
 // Workgroup b of a launch lands on XCD b % 8.  Re-number so that consecutive logical ids
 // (which share an expert's weights / an M-tile's rows) run on the same XCD and meet in its L2.
-__device__ __forceinline__ int64_t xcd_contiguous_id(int64_t block, int64_t n_blocks_padded) {
-  const int64_t per_xcd = n_blocks_padded / kNumXcd;
-  return (block % kNumXcd) * per_xcd + block / kNumXcd;
+// `n_tiles` is the number of tiles that really exist (the grid may be larger: its size is an
+// upper bound fixed on the host); the tiles are split evenly over the XCDs.  Returns -1 for a
+// workgroup without a tile.
+__device__ __forceinline__ int64_t xcd_contiguous_id(int64_t block, int64_t n_tiles) {
+  const int64_t per_xcd = (n_tiles + kNumXcd - 1) / kNumXcd;
+  const int64_t slot = block / kNumXcd;
+  if (slot >= per_xcd) return -1;
+  const int64_t id = (block % kNumXcd) * per_xcd + slot;
+  return id < n_tiles ? id : -1;
 }
 
 inline int64_t pad_to_xcd(int64_t n_blocks) { return (n_blocks + kNumXcd - 1) / kNumXcd * kNumXcd; }

@@ -143,7 +143,9 @@ __global__ __launch_bounds__(C::kThreads) void mfma_gemm_kernel(MfmaArgs p) {
   T* lds_b[2] = {smem + 2 * SA::kElems, smem + 2 * SA::kElems + SB::kElems};
 
   // ---- which tile is this workgroup's?
-  const int64_t id = xcd_contiguous_id(blockIdx.x, p.blocks_padded);
+  const int64_t n_tiles = WGRAD ? int64_t(p.n_groups) * p.tiles_i * p.tiles_j : int64_t(p.header[0]) * p.tiles_j;
+  const int64_t id = xcd_contiguous_id(blockIdx.x, n_tiles);
+  if (id < 0) return;
   const T* a = static_cast<const T*>(p.a);
   const T* b = static_cast<const T*>(p.b);
   T* c = static_cast<T*>(p.c);

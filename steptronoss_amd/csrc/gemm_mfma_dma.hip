@@ -1,33 +1,41 @@
-// bf16 / fp16 grouped GEMM, main kernels: buffer_load ... lds (HBM -> LDS without a register
-// stop), four LDS stages of 32 contraction elements, XOR-swizzled LDS rows, 32x32x16 MFMA.
+// bf16 / fp16 grouped GEMM, main kernels: persistent workgroups, buffer_load ... lds (HBM/L2 ->
+// LDS without a register stop), XOR-swizzled LDS tiles, 32x32x16 MFMA.
 //
-// Compared with the register-staged kernels of gemm_mfma.hip this keeps three stages of
-// loads in flight per workgroup (the latency of a load is covered by three compute steps
-// instead of one) and spends no VGPRs on staging.  The loads are raw buffer loads: anything
-// past the end of the operand's valid region (rows past a ragged group, rows past the tile
-// of a short M-tile) comes back as zero from the bounds check, so ragged edges need no
-// branches.  The same three products are covered as in gemm_mfma.hip:
+// Shape of the design (numbers for the 256 x 256 tile):
+//   * one workgroup of 4 waves per CU, resident for the whole launch; it walks a strided
+//     list of output tiles.  Tiles are numbered so that the workgroups of one XCD work on
+//     neighbouring tiles (same expert weights / same rows) and meet in that XCD's L2;
+//   * per contraction step of 64 elements each operand tile is 256 rows x 128 B.  Every
+//     wave-wide load instruction moves 8 full 128-byte lines (KC) or 2 x 512 contiguous bytes
+//     (KM) straight into LDS; two LDS stages of 64 KiB, the load of stage s+2 is issued as
+//     soon as the last wave has stopped reading stage s;
+//   * raw buffer loads: anything past the end of an operand's valid region (rows past a
+//     ragged group, rows past a short M-tile) reads as zero through the bounds check, so
+//     ragged edges cost no branches;
+//   * MFMA fragments are double-buffered in registers, the LDS reads of the next 16-wide
+//     slice are issued in the shadow of the current slice's MFMAs, also across stages and
+//     across tiles (the first loads of the next tile are issued before the epilogue of the
+//     current one).
 //
+// The three products of the expert FFN:
 //   fwd   C = A  * W^T   A:[M,K] KC   W[g]:[N,K] KC
 //   dgrad C = dY * W     dY:[M,K] KC  W[g]:[K,N] KM
 //   wgrad O = X^T * Y    X:[M,P] KM   Y:[M,Q] KM
+// KC = operand rows are contraction-contiguous (read with ds_read_b128),
+// KM = operand rows are contraction steps      (read with ds_read_b64_tr_b16).
 //
-// KC = rows of the operand are contraction-contiguous (read with ds_read_b128),
-// KM = rows of the operand are contraction steps   (read with ds_read_b64_tr_b16).
-//
-// LDS layout of one stage (BK = 32):
-//   KC tile: row r (64 B) at r*64, its four 16-byte chunks stored at chunk ^ ((r >> 2) & 3);
+// LDS layout of one stage:
+//   KC tile: row r (128 B) at r*128, its eight 16-byte chunks stored at chunk ^ ((r >> 1) & 7):
 //            16 consecutive rows read the same logical chunk from 16 distinct bank groups.
-//   KM tile: contraction row k (R*2 B) at k*R*2, its 64-byte chunks stored at chunk ^ (k & 3);
+//   KM tile: contraction row k (R*2 B) at k*R*2, its 64-byte chunks stored at chunk ^ (k & 3):
 //            the four rows a transposing read touches land in the four quarters of the banks.
 // A wave-wide buffer_load ... lds writes 1024 consecutive LDS bytes (lane l at +16*l), so the
 // swizzle is applied on the global-address side.
+#include <type_traits>
+
 #include "gemm_common.hpp"
 
 namespace stm {
-
-using DmaGemmArgs = GemmArgs;
-
 namespace {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -54,8 +62,8 @@ struct Mfma<f16_t> {
   }
 };
 
-constexpr int kBK = 32;
-constexpr int kStages = 4;
+constexpr int kBK = 64;      // contraction elements per stage
+constexpr int kStages = 2;
 constexpr int kThreads = 256;
 
 template <typename T>
@@ -67,9 +75,9 @@ struct alignas(sizeof(T) * 4) Pack4 {
 __device__ __forceinline__ i32x4_t make_rsrc(const void* base, uint32_t bytes) {
   const uint64_t p = reinterpret_cast<uint64_t>(base);
   i32x4_t r;
-  r[0] = int(uint32_t(p));
-  r[1] = int(uint32_t(p >> 32) & 0xffffu);  // stride 0
-  r[2] = int(bytes);
+  r[0] = __builtin_amdgcn_readfirstlane(int(uint32_t(p)));
+  r[1] = __builtin_amdgcn_readfirstlane(int(uint32_t(p >> 32) & 0xffffu));  // stride 0
+  r[2] = __builtin_amdgcn_readfirstlane(int(bytes));
   r[3] = 0x00020000;
   return r;
 }
@@ -89,55 +97,68 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-// Per-thread plan of one operand's loads for a stage: R/64 wave-loads per wave.
+// Per-thread plan of one operand's loads for a stage.  A stage is R*128 bytes = R/8 wave-wide
+// loads of 1 KiB; wave w issues loads w*L .. w*L+L-1 (L = kLoadsPerWave).  The byte offset of a
+// lane inside "its" load depends on the load index only through its parity (via the swizzle),
+// so two VGPRs per operand describe all of them; the first row of the load goes into the
+// scalar offset.
 template <int R, bool KM>
 struct OperandPlan {
-  static constexpr int kLoadsPerWave = R / 64;     // (R*64 B per stage) / 1024 B / 4 waves
   static constexpr int kStageBytes = R * kBK * 2;  // 16-bit elements
-  uint32_t voff[kLoadsPerWave];                    // byte offset of this lane's 16 bytes at step 0
-  uint32_t lds_off[kLoadsPerWave];                 // wave-uniform LDS offset of the wave-load
-  uint32_t step_bytes;                             // soffset increment per contraction step
+  static constexpr int kLoadsPerWave = kStageBytes / 1024 / (kThreads / kWave);
+  static constexpr int kRowsPerLoad = KM ? 1024 / (R * 2) : 8;  // stored rows covered by one load
+  static_assert(kLoadsPerWave % 2 == 0, "the parity trick needs an even number of loads per wave");
+  static_assert(!KM || kRowsPerLoad == 2 || kRowsPerLoad == 4, "KM tiles of 128 or 256 columns");
+  uint32_t voff[2];      // lane offset for even / odd loads, relative to the load's first row
+  uint32_t load_stride;  // bytes between the first rows of consecutive loads
+  uint32_t step_bytes;   // scalar offset increment per contraction step
 
-  __device__ __forceinline__ void init(int64_t ld_elems) {
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  __device__ __forceinline__ void init(int64_t ld_elems, int lane) {
+    const uint32_t row_bytes = uint32_t(ld_elems * 2);
 #pragma unroll
-    for (int j = 0; j < kLoadsPerWave; ++j) {
-      const int wl = wave * kLoadsPerWave + j;
-      lds_off[j] = uint32_t(wl) * 1024u;
+    for (int parity = 0; parity < 2; ++parity) {
       if constexpr (!KM) {
-        const int row = wl * 16 + lane / 4;
-        const int logical = (lane % 4) ^ (lane / 16);  // == phys ^ ((row >> 2) & 3)
-        voff[j] = uint32_t(row) * uint32_t(ld_elems * 2) + uint32_t(logical) * 16u;
+        // stored row r = load*8 + lane/8, chunk = (lane%8) ^ ((r >> 1) & 7)
+        const int sw = ((parity * 4) + lane / 16) & 7;
+        voff[parity] = uint32_t(lane / 8) * row_bytes + uint32_t((lane % 8) ^ sw) * 16u;
       } else {
-        constexpr int kChunks16 = R / 8;  // 16-byte chunks per stored row
-        constexpr int kRowsPerLoad = 64 / kChunks16;
-        const int row = wl * kRowsPerLoad + lane / kChunks16;
+        // stored row k = load*kRowsPerLoad + lane/(R/8), 64-byte chunk = (c16/4) ^ (k & 3)
+        constexpr int kChunks16 = R / 8;
+        const int row_in_load = lane / kChunks16;
         const int c16 = lane % kChunks16;
-        const int logical64 = (c16 / 4) ^ (row & 3);
-        const int col = logical64 * 32 + (c16 % 4) * 8;
-        voff[j] = uint32_t(row) * uint32_t(ld_elems * 2) + uint32_t(col) * 2u;
+        const int k_low = ((parity * kRowsPerLoad) + row_in_load) & 3;
+        const int col = (((c16 / 4) ^ k_low) * 32) + (c16 % 4) * 8;
+        voff[parity] = uint32_t(row_in_load) * row_bytes + uint32_t(col) * 2u;
       }
     }
-    step_bytes = KM ? uint32_t(kBK * ld_elems * 2) : uint32_t(kBK * 2);
+    load_stride = __builtin_amdgcn_readfirstlane(uint32_t(kRowsPerLoad) * row_bytes);
+    step_bytes = __builtin_amdgcn_readfirstlane(KM ? uint32_t(kBK) * row_bytes : uint32_t(kBK * 2));
   }
 
-  __device__ __forceinline__ void issue(i32x4_t rsrc, uint32_t lds_stage_addr, int step) const {
-    const uint32_t soff = __builtin_amdgcn_readfirstlane(uint32_t(step) * step_bytes);
+  __device__ __forceinline__ void issue(i32x4_t rsrc_in, uint32_t lds_stage_addr, int step, int wave) const {
+    i32x4_t rsrc;  // the descriptor must sit in SGPRs whatever path it took to get here
+#pragma unroll
+    for (int w = 0; w < 4; ++w) rsrc[w] = __builtin_amdgcn_readfirstlane(rsrc_in[w]);
+    const uint32_t first = uint32_t(wave * kLoadsPerWave);
+    uint32_t soff = __builtin_amdgcn_readfirstlane(uint32_t(step) * step_bytes + first * load_stride);
+    asm volatile("" : "+s"(soff));  // keep it in an SGPR: a folded literal is not a legal soffset
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_stage_addr + first * 1024u);
 #pragma unroll
     for (int j = 0; j < kLoadsPerWave; ++j)
-      dma16(rsrc, __builtin_amdgcn_readfirstlane(lds_stage_addr + lds_off[j]), voff[j], soff);
+      dma16(rsrc, lds0 + uint32_t(j) * 1024u, voff[j & 1], soff + uint32_t(j) * load_stride);
   }
 };
 
 // 8 contraction values (k = kk*16 + (lane/32)*8 .. +8) of output row/column r0 + lane%32.
 template <int R, bool KM>
-__device__ __forceinline__ uint4 read_fragment(const unsigned char* tile, int r0, int kk) {
-  const int lane = threadIdx.x % kWave;
+__device__ __forceinline__ uint4 read_fragment(const unsigned char* tile, int r0, int kk, int lane) {
   if constexpr (!KM) {
     const int r = r0 + lane % 32;
-    const int chunk = (kk * 2 + lane / 32) ^ ((r >> 2) & 3);
-    return *reinterpret_cast<const uint4*>(tile + r * 64 + chunk * 16);
+    const int chunk = (kk * 2 + lane / 32) ^ ((r >> 1) & 7);
+    return *reinterpret_cast<const uint4*>(tile + r * 128 + chunk * 16);
   } else {
+    // in each 16-lane group, lanes 4r..4r+3 name stored row r (4 elements each) and lane i
+    // receives column i of those four rows
     const int i = lane % 16;
     const int col = r0 + ((lane / 16) & 1) * 16 + 4 * (i % 4);
     const int row = kk * 16 + (lane / 32) * 8 + i / 4;  // second read: row + 4 (same row & 3)
@@ -150,8 +171,15 @@ __device__ __forceinline__ uint4 read_fragment(const unsigned char* tile, int r0
   }
 }
 
+template <typename T>
+struct TileState {
+  i32x4_t rsrc_a, rsrc_b;
+  T* c;
+  int valid_i, valid_j, n_steps;
+};
+
 template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD>
-__global__ __launch_bounds__(kThreads) void dma_gemm_kernel(DmaGemmArgs p) {
+__global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
   constexpr int TM = BM / 64, TN = BN / 64;  // 32x32 MFMA tiles per wave (waves are laid out 2 x 2)
   using PlanA = OperandPlan<BM, A_KM>;
   using PlanB = OperandPlan<BN, B_KM>;
@@ -159,138 +187,259 @@ __global__ __launch_bounds__(kThreads) void dma_gemm_kernel(DmaGemmArgs p) {
   constexpr int kLoadsPerStep = PlanA::kLoadsPerWave + PlanB::kLoadsPerWave;
   extern __shared__ __align__(1024) unsigned char smem[];
 
-  // ---- which tile is this workgroup's?
-  const int64_t id = xcd_contiguous_id(blockIdx.x, p.blocks_padded);
-  const T* a = static_cast<const T*>(p.a);
-  const T* b = static_cast<const T*>(p.b);
-  T* c = static_cast<T*>(p.c);
-  int valid_i, valid_j, n_k;
-  uint32_t a_bytes, b_bytes;
-  const int jt = int(id % p.tiles_j);
-  const int j0 = jt * BN;
-  valid_j = p.n_j - j0;
-  if constexpr (WGRAD) {
-    const int64_t rest = id / p.tiles_j;
-    const int it = int(rest % p.tiles_i);
-    const int64_t g = rest / p.tiles_i;
-    if (g >= p.n_groups) return;
-    const int64_t lo = p.offsets[g], hi = p.offsets[g + 1];
-    n_k = hi > lo ? int(hi - lo) : 0;
-    const int i0 = it * BM;
-    valid_i = p.n_i - i0;
-    a += lo * p.lda + i0;
-    b += lo * p.ldb + j0;
-    c += g * p.c_group + int64_t(i0) * p.ldc + j0;
-    // contraction rows past the end of the group are past the end of the buffer: zeros
-    a_bytes = uint32_t(int64_t(n_k) * p.lda * 2 - int64_t(i0) * 2);
-    b_bytes = uint32_t(int64_t(n_k) * p.ldb * 2 - int64_t(j0) * 2);
-  } else {
-    const int64_t mt = id / p.tiles_j;
-    if (mt >= p.header[0]) return;
-    const MTile t = p.tiles[mt];
-    n_k = p.n_k;
-    valid_i = t.rows;
-    a += int64_t(t.row0) * p.lda;
-    c += int64_t(t.row0) * p.ldc + j0;
-    a_bytes = uint32_t(int64_t(t.rows) * p.lda * 2);
-    if constexpr (B_KM) {
-      b += int64_t(t.group) * p.b_group + j0;
-      b_bytes = uint32_t(int64_t(p.n_k) * p.ldb * 2 - int64_t(j0) * 2);
+  // ---- this workgroup's tiles: XCD x = blockIdx % 8 owns tiles [x*per_xcd, (x+1)*per_xcd);
+  // its workgroups take them round-robin, so that at any time they sit next to each other.
+  const int64_t n_tiles = WGRAD ? int64_t(p.n_groups) * p.tiles_i * p.tiles_j : int64_t(p.header[0]) * p.tiles_j;
+  const int64_t per_xcd = (n_tiles + kNumXcd - 1) / kNumXcd;
+  const int64_t xcd = blockIdx.x % kNumXcd;
+  const int64_t wgs_per_xcd = gridDim.x / kNumXcd;
+  auto tile_id = [&](int64_t k) -> int64_t {
+    if (k >= per_xcd) return -1;
+    const int64_t id = xcd * per_xcd + k;
+    return id < n_tiles ? id : -1;
+  };
+  auto locate = [&](int64_t id, TileState<T>& t) {
+    const T* a = static_cast<const T*>(p.a);
+    const T* b = static_cast<const T*>(p.b);
+    T* c = static_cast<T*>(p.c);
+    const int jt = int(id % p.tiles_j);
+    const int j0 = jt * BN;
+    int n_k;
+    uint32_t a_bytes, b_bytes;
+    t.valid_j = p.n_j - j0;
+    if constexpr (WGRAD) {
+      const int64_t rest = id / p.tiles_j;
+      const int it = int(rest % p.tiles_i);
+      const int64_t g = rest / p.tiles_i;
+      const int64_t lo = p.offsets[g], hi = p.offsets[g + 1];
+      n_k = hi > lo ? int(hi - lo) : 0;
+      const int i0 = it * BM;
+      t.valid_i = p.n_i - i0;
+      a += lo * p.lda + i0;
+      b += lo * p.ldb + j0;
+      c += g * p.c_group + int64_t(i0) * p.ldc + j0;
+      // contraction rows past the end of the group are past the end of the buffer: zeros
+      a_bytes = uint32_t(int64_t(n_k) * p.lda * 2 - int64_t(i0) * 2);
+      b_bytes = uint32_t(int64_t(n_k) * p.ldb * 2 - int64_t(j0) * 2);
     } else {
-      b += int64_t(t.group) * p.b_group + int64_t(j0) * p.ldb;
-      b_bytes = uint32_t(int64_t(valid_j < BN ? valid_j : BN) * p.ldb * 2);
+      const MTile mt = p.tiles[id / p.tiles_j];
+      n_k = p.n_k;
+      t.valid_i = mt.rows;
+      a += int64_t(mt.row0) * p.lda;
+      c += int64_t(mt.row0) * p.ldc + j0;
+      a_bytes = uint32_t(int64_t(mt.rows) * p.lda * 2);
+      if constexpr (B_KM) {
+        b += int64_t(mt.group) * p.b_group + j0;
+        b_bytes = uint32_t(int64_t(p.n_k) * p.ldb * 2 - int64_t(j0) * 2);
+      } else {
+        b += int64_t(mt.group) * p.b_group + int64_t(j0) * p.ldb;
+        b_bytes = uint32_t(int64_t(t.valid_j < BN ? t.valid_j : BN) * p.ldb * 2);
+      }
     }
-  }
-  i32x4_t rsrc_a = make_rsrc(a, a_bytes);
-  i32x4_t rsrc_b = make_rsrc(b, b_bytes);
-#pragma unroll
-  for (int w = 0; w < 4; ++w) {
-    rsrc_a[w] = __builtin_amdgcn_readfirstlane(rsrc_a[w]);
-    rsrc_b[w] = __builtin_amdgcn_readfirstlane(rsrc_b[w]);
-  }
+    t.rsrc_a = make_rsrc(a, a_bytes);
+    t.rsrc_b = make_rsrc(b, b_bytes);
+    t.c = c;
+    t.n_steps = __builtin_amdgcn_readfirstlane((n_k + kBK - 1) / kBK);
+  };
 
   PlanA plan_a;
   PlanB plan_b;
-  plan_a.init(p.lda);
-  plan_b.init(p.ldb);
   const uint32_t lds_base =
       uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)smem));  // LDS offset
-
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int lane = threadIdx.x % kWave;
-  const int wave_i = (wave / 2) * (BM / 2);
+  plan_a.init(p.lda, lane);
+  plan_b.init(p.ldb, lane);
+  auto issue = [&](const TileState<T>& t, int step) {
+    const uint32_t stage = lds_base + uint32_t(step % kStages) * kStageBytes;
+    plan_a.issue(t.rsrc_a, stage, step, wave);
+    plan_b.issue(t.rsrc_b, stage + PlanA::kStageBytes, step, wave);
+  };
+
+  // Along M the 32-row sub-blocks of the tile are dealt to the two wave rows alternately (wave
+  // row w owns sub-blocks w, w+2, ...), so that a short M-tile (the ragged tail of an expert)
+  // leaves both wave rows with about half of its live sub-blocks; the contraction code is
+  // specialised on the number of live sub-blocks of the wave.
+  const int wave_row = wave / 2;
   const int wave_j = (wave % 2) * (BN / 2);
 
-  f32x16_t acc[TM][TN];
+  // One tile: `cur` has its first stage (two, if it has two) in flight on entry; on exit the
+  // same holds for `next` (if next_id >= 0).
+  auto run_tile = [&](auto atm_tag, const TileState<T>& cur, int64_t next_id, TileState<T>& next) {
+    constexpr int ATM = decltype(atm_tag)::value;
+    constexpr int AR = ATM > 0 ? ATM : 1;
+    // The lane index as seen by this tile's address arithmetic: passed through an opaque asm so
+    // that the (many) LDS addresses derived from it are recomputed per tile instead of being
+    // hoisted out of the tile loop, where they would crowd the accumulators out of registers.
+    int tl = lane;
+    asm volatile("" : "+v"(tl));
+    f32x16_t acc[AR][TN];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < AR; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    uint4 fa[2][AR], fb[2][TN];
+    auto read_set = [&](int set, int step, int kk) {
+      const unsigned char* ta = smem + (step % kStages) * kStageBytes;
+      const unsigned char* tb = ta + PlanA::kStageBytes;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[set][j] = read_fragment<BN, B_KM>(tb, wave_j + j * 32, kk, tl);
+#pragma unroll
+      for (int i = 0; i < ATM; ++i) fa[set][i] = read_fragment<BM, A_KM>(ta, (2 * i + wave_row) * 32, kk, tl);
+    };
+    auto mma_set = [&](int set) {
+#pragma unroll
+      for (int i = 0; i < ATM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(fb[set][j], fa[set][i], acc[i][j]);
+    };
+    // scheduling hint: LDS reads in the shadow of the MFMAs
+    auto interleave = [&]() {
+      constexpr int kReads = (TN * (B_KM ? 2 : 1) + ATM * (A_KM ? 2 : 1));
+      constexpr int kMfma = ATM * TN;
+      if constexpr (kMfma > 0) {
+#pragma unroll
+        for (int r = 0; r < kReads; ++r) {
+          __builtin_amdgcn_sched_group_barrier(0x008, (kMfma >= 2 * kReads) ? 2 : 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+      }
+    };
+    auto prefetch_next = [&]() {
+      if (next_id >= 0) {
+        locate(next_id, next);
+        if (next.n_steps > 0) issue(next, 0);
+      }
+    };
 
-  const int n_steps = (n_k + kBK - 1) / kBK;
-  auto issue = [&](int step) {
-    const uint32_t stage = lds_base + uint32_t(step % kStages) * kStageBytes;
-    plan_a.issue(rsrc_a, stage, step);
-    plan_b.issue(rsrc_b, stage + PlanA::kStageBytes, step);
-  };
-#pragma unroll
-  for (int s = 0; s < kStages - 1; ++s)
-    if (s < n_steps) issue(s);
-
-  for (int step = 0; step < n_steps; ++step) {
-    // loads of stages step+1, step+2 may stay in flight; everything older must have landed
-    const int later = n_steps - 1 - step;
-    if (later >= 2)
-      wait_vmcnt<2 * kLoadsPerStep>();
-    else if (later == 1)
-      wait_vmcnt<kLoadsPerStep>();
-    else
-      wait_vmcnt<0>();
-    __syncthreads();  // every wave's part of this stage is in LDS; stage (step-1) is free again
-    if (step + kStages - 1 < n_steps) issue(step + kStages - 1);
-    const unsigned char* ta = smem + (step % kStages) * kStageBytes;
-    const unsigned char* tb = ta + PlanA::kStageBytes;
-#pragma unroll
-    for (int kk = 0; kk < kBK / 16; ++kk) {
-      uint4 fa[TM], fb[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) fa[i] = read_fragment<BM, A_KM>(ta, wave_i + i * 32, kk);
-#pragma unroll
-      for (int j = 0; j < TN; ++j) fb[j] = read_fragment<BN, B_KM>(tb, wave_j + j * 32, kk);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
+    const int n_steps = __builtin_amdgcn_readfirstlane(cur.n_steps);  // wave-uniform: scalar branches
+    if (n_steps > 0) {
+      // stage 0 has landed when at most the loads of stage 1 are outstanding (the stores of the
+      // previous tile's epilogue were issued between the two and are then done as well)
+      if (n_steps > 1)
+        wait_vmcnt<kLoadsPerStep>();
+      else
+        wait_vmcnt<0>();
+      __syncthreads();
+      read_set(0, 0, 0);
+      for (int step = 0; step + 1 < n_steps; ++step) {
+        read_set(1, step, 1);
+        mma_set(0);
+        interleave();
+        read_set(0, step, 2);
+        mma_set(1);
+        interleave();
+        read_set(1, step, 3);
+        mma_set(0);
+        interleave();
+        wait_vmcnt<0>();                                    // stage step+1 has landed (my part)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // my reads of stage `step` are done
+        __syncthreads();  // stage step+1 is complete in LDS and nobody reads stage `step` any more
+        if (step + kStages < n_steps) issue(cur, step + kStages);  // refill the slot of stage `step`
+        read_set(0, step + 1, 0);
+        mma_set(1);
+        interleave();
+      }
+      const int last = n_steps - 1;
+      read_set(1, last, 1);
+      mma_set(0);
+      interleave();
+      read_set(0, last, 2);
+      mma_set(1);
+      interleave();
+      read_set(1, last, 3);
+      mma_set(0);
+      interleave();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __syncthreads();  // both stages are free: the next tile may start to arrive
+      prefetch_next();
+      mma_set(1);
+    } else {
+      __syncthreads();
+      prefetch_next();
     }
-  }
-
-  // ---- epilogue: lane owns row (lane % 32) and, per group of four registers, four
-  // consecutive columns starting at (r/4)*8 + (lane/32)*4.
+    // ---- epilogue.  In the accumulators a lane owns row (lane % 32) of a sub-block and, per
+    // group of four registers, four consecutive columns starting at (r/4)*8 + (lane/32)*4:
+    // stored from there, a wave-wide store would touch 32 rows with 16 bytes each.  Instead a
+    // 32 x 128 sub-block is rounded, written to LDS (16-byte chunks XOR-swizzled with the row)
+    // and read back row-wise, so that every store instruction writes four full 256-byte row
+    // segments.  The scratch is the part of the second LDS stage this very wave refills
+    // afterwards, so no other wave is involved and no workgroup barrier is needed.
+    static_assert(BN == 256 && sizeof(T) == 2, "epilogue staging assumes 128 columns of 16-bit outputs per wave");
+    unsigned char* scratch[2] = {smem + kStageBytes + wave * 8192,
+                                 smem + kStageBytes + PlanA::kStageBytes + wave * 8192};
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int row = wave_i + i * 32 + lane % 32;
-    if (row >= valid_i) continue;
-    T* crow = c + int64_t(row) * p.ldc;
+    for (int i = 0; i < ATM; ++i) {
+      unsigned char* buf = scratch[i & 1];
+      const int r = tl % 32;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
+      for (int j = 0; j < TN; ++j) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int col = wave_j + j * 32 + q * 8 + (lane / 32) * 4;
-        if (col >= valid_j) continue;
-        Pack4<T> out;
+        for (int q = 0; q < 4; ++q) {
+          Pack4<T> out;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) out.v[e] = from_float<T>(acc[i][j][q * 4 + e]);
-        *reinterpret_cast<Pack4<T>*>(crow + col) = out;
+          for (int e = 0; e < 4; ++e) out.v[e] = from_float<T>(acc[i][j][q * 4 + e]);
+          const int chunk = (j * 4 + q) ^ (r & 15);
+          *reinterpret_cast<Pack4<T>*>(buf + r * 256 + chunk * 16 + (tl / 32) * 8) = out;
+        }
+      }
+      const int row0 = (2 * i + wave_row) * 32;
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int id = it * kWave + tl;
+        const int row = id / 16, c16 = id % 16;
+        const uint4 v = *reinterpret_cast<const uint4*>(buf + row * 256 + ((c16 ^ (row & 15)) * 16));
+        const int col = wave_j + c16 * 8;
+        if (row0 + row < cur.valid_i && col < cur.valid_j)
+          *reinterpret_cast<uint4*>(cur.c + int64_t(row0 + row) * p.ldc + col) = v;
       }
     }
+    // the second stage of the next tile goes out behind the stores (see the wait above)
+    if (next_id >= 0 && __builtin_amdgcn_readfirstlane(next.n_steps) > 1) issue(next, 1);
+  };
+
+  int64_t k = blockIdx.x / kNumXcd;
+  int64_t id = tile_id(k);
+  if (id < 0) return;
+  TileState<T> cur, next;
+  locate(id, cur);
+  if (cur.n_steps > 0) issue(cur, 0);
+  if (cur.n_steps > 1) issue(cur, 1);
+  while (true) {
+    const int64_t next_id = tile_id(k + wgs_per_xcd);
+    const int live_sub = (cur.valid_i < BM ? cur.valid_i + 31 : BM) / 32;  // live 32-row sub-blocks
+    const int my_sub = __builtin_amdgcn_readfirstlane((live_sub + 1 - wave_row) / 2);  // those of this wave row
+    switch (my_sub) {
+      case 0: run_tile(std::integral_constant<int, 0>{}, cur, next_id, next); break;
+      case 1: run_tile(std::integral_constant<int, 1>{}, cur, next_id, next); break;
+      case 2: run_tile(std::integral_constant<int, (TM >= 2 ? 2 : TM)>{}, cur, next_id, next); break;
+      case 3: run_tile(std::integral_constant<int, (TM >= 3 ? 3 : TM)>{}, cur, next_id, next); break;
+      default: run_tile(std::integral_constant<int, TM>{}, cur, next_id, next); break;
+    }
+    if (next_id < 0) break;
+    cur = next;
+    k += wgs_per_xcd;
   }
 }
 
+int persistent_grid() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    cached = cus / kNumXcd * kNumXcd;
+    if (cached < kNumXcd) cached = kNumXcd;
+  }
+  return cached;
+}
+
 template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD>
-int launch(const DmaGemmArgs& p, int64_t n_blocks, hipStream_t s) {
-  auto kernel = dma_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD>;
+int launch(const GemmArgs& p, hipStream_t s) {
+  auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD>;
   constexpr size_t smem = size_t(kStages) * (BM + BN) * kBK * 2;
   static bool configured = false;
   if (!configured) {
@@ -299,9 +448,7 @@ int launch(const DmaGemmArgs& p, int64_t n_blocks, hipStream_t s) {
       return STM_ERR_LAUNCH;
     configured = true;
   }
-  DmaGemmArgs q = p;
-  q.blocks_padded = pad_to_xcd(n_blocks);
-  kernel<<<unsigned(q.blocks_padded), kThreads, smem, s>>>(q);
+  kernel<<<unsigned(persistent_grid()), kThreads, smem, s>>>(p);
   return launch_status();
 }
 
@@ -310,32 +457,31 @@ int launch(const DmaGemmArgs& p, int64_t n_blocks, hipStream_t s) {
 constexpr int kDmaBM = 256, kDmaBN = 256;
 
 // rows form; returns STM_ERR_UNSUPPORTED when the shape does not fit these kernels.
-int launch_dma_rows(int dtype, const DmaGemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap,
-                    int b_is_nk, void* ws, hipStream_t s) {
-  DmaGemmArgs p = base;
+int launch_dma_rows(int dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap, int b_is_nk,
+                    void* ws, hipStream_t s) {
+  GemmArgs p = base;
   if (p.n_k % kBK != 0 || p.n_j % 8 != 0) return STM_ERR_UNSUPPORTED;
   if (int64_t(p.n_k) * p.ldb * 2 >= (int64_t(1) << 32) || int64_t(kDmaBM) * p.lda * 2 >= (int64_t(1) << 32))
     return STM_ERR_UNSUPPORTED;
   const int st = build_tile_table(offsets, n_groups, kDmaBM, m_cap, ws, s);
   if (st != STM_OK) return st;
   p.tiles_j = (p.n_j + kDmaBN - 1) / kDmaBN;
-  const int64_t blocks = max_m_tiles(m_cap, n_groups, kDmaBM) * p.tiles_j;
   if (dtype == STM_BF16)
-    return b_is_nk ? launch<bf16_t, kDmaBM, kDmaBN, false, false, false>(p, blocks, s)
-                   : launch<bf16_t, kDmaBM, kDmaBN, false, true, false>(p, blocks, s);
-  return b_is_nk ? launch<f16_t, kDmaBM, kDmaBN, false, false, false>(p, blocks, s)
-                 : launch<f16_t, kDmaBM, kDmaBN, false, true, false>(p, blocks, s);
+    return b_is_nk ? launch<bf16_t, kDmaBM, kDmaBN, false, false, false>(p, s)
+                   : launch<bf16_t, kDmaBM, kDmaBN, false, true, false>(p, s);
+  return b_is_nk ? launch<f16_t, kDmaBM, kDmaBN, false, false, false>(p, s)
+                 : launch<f16_t, kDmaBM, kDmaBN, false, true, false>(p, s);
 }
 
-int launch_dma_wgrad(int dtype, const DmaGemmArgs& base, int n_groups, int64_t m_cap, hipStream_t s) {
-  DmaGemmArgs p = base;
+int launch_dma_wgrad(int dtype, const GemmArgs& base, int n_groups, int64_t m_cap, hipStream_t s) {
+  GemmArgs p = base;
   if (p.n_i % 8 != 0 || p.n_j % 8 != 0) return STM_ERR_UNSUPPORTED;
   if (m_cap * p.lda * 2 >= (int64_t(1) << 32) || m_cap * p.ldb * 2 >= (int64_t(1) << 32)) return STM_ERR_UNSUPPORTED;
   p.tiles_i = (p.n_i + kDmaBM - 1) / kDmaBM;
   p.tiles_j = (p.n_j + kDmaBN - 1) / kDmaBN;
-  const int64_t blocks = int64_t(n_groups) * p.tiles_i * p.tiles_j;
-  if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, true, true, true>(p, blocks, s);
-  return launch<f16_t, kDmaBM, kDmaBN, true, true, true>(p, blocks, s);
+  p.n_groups = n_groups;
+  if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, true, true, true>(p, s);
+  return launch<f16_t, kDmaBM, kDmaBN, true, true, true>(p, s);
 }
 
 }  // namespace stm
