@@ -1,21 +1,23 @@
 // bf16 / fp16 grouped GEMM, main kernels: persistent workgroups, buffer_load ... lds (HBM/L2 ->
 // LDS without a register stop), XOR-swizzled LDS tiles, 32x32x16 MFMA.
 //
-// Shape of the design (numbers for the 256 x 256 tile):
-//   * one workgroup of 4 waves per CU, resident for the whole launch; it walks a strided
-//     list of output tiles.  Tiles are numbered so that the workgroups of one XCD work on
-//     neighbouring tiles (same expert weights / same rows) and meet in that XCD's L2;
-//   * per contraction step of 64 elements each operand tile is 256 rows x 128 B.  Every
-//     wave-wide load instruction moves 8 full 128-byte lines (KC) or 2 x 512 contiguous bytes
-//     (KM) straight into LDS; two LDS stages of 64 KiB, the load of stage s+2 is issued as
-//     soon as the last wave has stopped reading stage s;
-//   * raw buffer loads: anything past the end of an operand's valid region (rows past a
-//     ragged group, rows past a short M-tile) reads as zero through the bounds check, so
-//     ragged edges cost no branches;
-//   * MFMA fragments are double-buffered in registers, the LDS reads of the next 16-wide
-//     slice are issued in the shadow of the current slice's MFMAs, also across stages and
-//     across tiles (the first loads of the next tile are issued before the epilogue of the
-//     current one).
+// Shape of the design (256 x 256 output tile, contraction step 64):
+//   * one workgroup of 4 waves per CU, resident for the whole launch, walks a strided list of
+//     output tiles.  Tiles are numbered so that the workgroups of one XCD work on neighbouring
+//     tiles (same expert weights / same rows) and meet in that XCD's L2;
+//   * per step each operand tile is 256 rows x 128 B; a wave-wide load instruction moves 8 full
+//     128-byte lines (KC) or 2 x 512 contiguous bytes (KM) straight into LDS.  The CU's texture
+//     path takes about 64 cycles per such instruction, i.e. about half of a step's MFMA time
+//     for the 64 loads of a stage -- so the loads are not issued in a burst but one at a time
+//     in the shadow of the MFMAs, spread over three quarters of a step;
+//   * two LDS stages.  The (tile, step) pairs of a workgroup form ONE stream of stages: the
+//     loads of stage g+2 start as soon as every wave has read stage g, whether or not g+2
+//     belongs to the next tile, and the first MFMA fragments of a tile are fetched during the
+//     last MFMAs of the previous one; the epilogue runs while the next tile's data arrives;
+//   * raw buffer loads: anything past the end of an operand's valid region (rows past a ragged
+//     group, rows past a short M-tile) reads as zero through the bounds check, so ragged edges
+//     cost no branches;
+//   * MFMA fragments are double-buffered in registers, one LDS read per two MFMAs.
 //
 // The three products of the expert FFN:
 //   fwd   C = A  * W^T   A:[M,K] KC   W[g]:[N,K] KC
@@ -43,6 +45,7 @@ typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef int i32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr;
 
 template <typename T>
@@ -62,9 +65,10 @@ struct Mfma<f16_t> {
   }
 };
 
-constexpr int kBK = 64;      // contraction elements per stage
+constexpr int kBK = 64;  // contraction elements per stage
 constexpr int kStages = 2;
 constexpr int kThreads = 256;
+constexpr int kEpilogueScratch = 8192;  // bytes per wave, behind the stages
 
 template <typename T>
 struct alignas(sizeof(T) * 4) Pack4 {
@@ -90,11 +94,6 @@ __device__ __forceinline__ void dma16(i32x4_t rsrc, uint32_t lds_addr, uint32_t 
       :
       : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
       : "memory");
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
 // Per-thread plan of one operand's loads for a stage.  A stage is R*128 bytes = R/8 wave-wide
@@ -135,17 +134,20 @@ struct OperandPlan {
     step_bytes = __builtin_amdgcn_readfirstlane(KM ? uint32_t(kBK) * row_bytes : uint32_t(kBK * 2));
   }
 
-  __device__ __forceinline__ void issue(i32x4_t rsrc_in, uint32_t lds_stage_addr, int step, int wave) const {
-    i32x4_t rsrc;  // the descriptor must sit in SGPRs whatever path it took to get here
+  // scalar offset of this wave's first load of contraction step `step`
+  __device__ __forceinline__ uint32_t stage_soffset(int step, int wave) const {
+    return __builtin_amdgcn_readfirstlane(uint32_t(step) * step_bytes + uint32_t(wave * kLoadsPerWave) * load_stride);
+  }
+  // load j (0 <= j < kLoadsPerWave) of this wave; everything but the lane offset is scalar
+  // (the readfirstlane calls fold away when the value already sits in a scalar register; they
+  // are the guarantee the inline asm needs when it does not)
+  __device__ __forceinline__ void issue_one(i32x4_t rsrc_in, uint32_t lds_wave_addr, uint32_t soff0, int j) const {
+    i32x4_t rsrc;
 #pragma unroll
     for (int w = 0; w < 4; ++w) rsrc[w] = __builtin_amdgcn_readfirstlane(rsrc_in[w]);
-    const uint32_t first = uint32_t(wave * kLoadsPerWave);
-    uint32_t soff = __builtin_amdgcn_readfirstlane(uint32_t(step) * step_bytes + first * load_stride);
+    uint32_t soff = __builtin_amdgcn_readfirstlane(soff0 + uint32_t(j) * load_stride);
     asm volatile("" : "+s"(soff));  // keep it in an SGPR: a folded literal is not a legal soffset
-    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_stage_addr + first * 1024u);
-#pragma unroll
-    for (int j = 0; j < kLoadsPerWave; ++j)
-      dma16(rsrc, lds0 + uint32_t(j) * 1024u, voff[j & 1], soff + uint32_t(j) * load_stride);
+    dma16(rsrc, __builtin_amdgcn_readfirstlane(lds_wave_addr + uint32_t(j) * 1024u), voff[j & 1], soff);
   }
 };
 
@@ -184,12 +186,22 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
   using PlanA = OperandPlan<BM, A_KM>;
   using PlanB = OperandPlan<BN, B_KM>;
   constexpr uint32_t kStageBytes = PlanA::kStageBytes + PlanB::kStageBytes;
-  constexpr int kLoadsPerStep = PlanA::kLoadsPerWave + PlanB::kLoadsPerWave;
+  constexpr int kLoadsA = PlanA::kLoadsPerWave, kLoadsB = PlanB::kLoadsPerWave;
+  constexpr int kLoads = kLoadsA + kLoadsB;  // per wave per stage
+  // where in a step the loads of later stages go out: the first kEarly loads of stage g+2 in the
+  // last quarter of step g (right after its slot is free), the rest in the first two quarters
+  // of step g+1; they have landed when step g+1 reaches its third quarter.
+  constexpr int kEarly = kLoads * 3 / 8;
+  constexpr int kMid = kEarly + (kLoads - kEarly + 1) / 2;
+  static_assert(BN == 256 && sizeof(T) == 2, "epilogue staging assumes 128 columns of 16-bit outputs per wave");
   extern __shared__ __align__(1024) unsigned char smem[];
 
   // ---- this workgroup's tiles: XCD x = blockIdx % 8 owns tiles [x*per_xcd, (x+1)*per_xcd);
   // its workgroups take them round-robin, so that at any time they sit next to each other.
-  const int64_t n_tiles = WGRAD ? int64_t(p.n_groups) * p.tiles_i * p.tiles_j : int64_t(p.header[0]) * p.tiles_j;
+  // (values loaded from memory are pinned to scalar registers at once: all tile bookkeeping
+  // below is wave-uniform and must stay on the scalar unit)
+  const int64_t n_tiles = WGRAD ? int64_t(p.n_groups) * p.tiles_i * p.tiles_j
+                                : int64_t(__builtin_amdgcn_readfirstlane(p.header[0])) * p.tiles_j;
   const int64_t per_xcd = (n_tiles + kNumXcd - 1) / kNumXcd;
   const int64_t xcd = blockIdx.x % kNumXcd;
   const int64_t wgs_per_xcd = gridDim.x / kNumXcd;
@@ -211,7 +223,8 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
       const int64_t rest = id / p.tiles_j;
       const int it = int(rest % p.tiles_i);
       const int64_t g = rest / p.tiles_i;
-      const int64_t lo = p.offsets[g], hi = p.offsets[g + 1];
+      const int64_t lo = __builtin_amdgcn_readfirstlane(p.offsets[g]);
+      const int64_t hi = __builtin_amdgcn_readfirstlane(p.offsets[g + 1]);
       n_k = hi > lo ? int(hi - lo) : 0;
       const int i0 = it * BM;
       t.valid_i = p.n_i - i0;
@@ -219,10 +232,15 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
       b += lo * p.ldb + j0;
       c += g * p.c_group + int64_t(i0) * p.ldc + j0;
       // contraction rows past the end of the group are past the end of the buffer: zeros
-      a_bytes = uint32_t(int64_t(n_k) * p.lda * 2 - int64_t(i0) * 2);
-      b_bytes = uint32_t(int64_t(n_k) * p.ldb * 2 - int64_t(j0) * 2);
+      const int64_t ab = int64_t(n_k) * p.lda * 2 - int64_t(i0) * 2;
+      const int64_t bb = int64_t(n_k) * p.ldb * 2 - int64_t(j0) * 2;
+      a_bytes = ab > 0 ? uint32_t(ab) : 0u;
+      b_bytes = bb > 0 ? uint32_t(bb) : 0u;
     } else {
-      const MTile mt = p.tiles[id / p.tiles_j];
+      MTile mt = p.tiles[id / p.tiles_j];
+      mt.group = __builtin_amdgcn_readfirstlane(mt.group);
+      mt.row0 = __builtin_amdgcn_readfirstlane(mt.row0);
+      mt.rows = __builtin_amdgcn_readfirstlane(mt.rows);
       n_k = p.n_k;
       t.valid_i = mt.rows;
       a += int64_t(mt.row0) * p.lda;
@@ -239,23 +257,19 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
     t.rsrc_a = make_rsrc(a, a_bytes);
     t.rsrc_b = make_rsrc(b, b_bytes);
     t.c = c;
-    t.n_steps = __builtin_amdgcn_readfirstlane((n_k + kBK - 1) / kBK);
+    // an empty group still gets one step: all of its loads are out of bounds, i.e. zeros
+    const int steps = (n_k + kBK - 1) / kBK;
+    t.n_steps = __builtin_amdgcn_readfirstlane(steps > 0 ? steps : 1);
   };
 
-  PlanA plan_a;
-  PlanB plan_b;
-  const uint32_t lds_base =
-      uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)smem));  // LDS offset
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int lane = threadIdx.x % kWave;
+  PlanA plan_a;
+  PlanB plan_b;
   plan_a.init(p.lda, lane);
   plan_b.init(p.ldb, lane);
-  auto issue = [&](const TileState<T>& t, int step) {
-    const uint32_t stage = lds_base + uint32_t(step % kStages) * kStageBytes;
-    plan_a.issue(t.rsrc_a, stage, step, wave);
-    plan_b.issue(t.rsrc_b, stage + PlanA::kStageBytes, step, wave);
-  };
-
+  const uint32_t lds_base =
+      uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)smem));  // LDS offset
   // Along M the 32-row sub-blocks of the tile are dealt to the two wave rows alternately (wave
   // row w owns sub-blocks w, w+2, ...), so that a short M-tile (the ragged tail of an expert)
   // leaves both wave rows with about half of its live sub-blocks; the contraction code is
@@ -263,9 +277,66 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
   const int wave_row = wave / 2;
   const int wave_j = (wave % 2) * (BN / 2);
 
-  // One tile: `cur` has its first stage (two, if it has two) in flight on entry; on exit the
-  // same holds for `next` (if next_id >= 0).
-  auto run_tile = [&](auto atm_tag, const TileState<T>& cur, int64_t next_id, TileState<T>& next) {
+  // ---- the load cursor: walks the stream of stages ahead of the MFMAs.  Its state is
+  // wave-uniform (scalar registers).  Moving to the next step of a tile costs a handful of
+  // scalar adds; only a change of tile runs the tile lookup.  Past the last tile the cursor
+  // keeps going with an empty descriptor: such loads move no data (and write zeros to an LDS
+  // slot nobody reads any more), which keeps the steady-state code free of branches.
+  i32x4_t l_rsrc_a, l_rsrc_b;
+  const uint32_t l_soff_a0 = plan_a.stage_soffset(0, wave), l_soff_b0 = plan_b.stage_soffset(0, wave);
+  const uint32_t l_lds_a0 = __builtin_amdgcn_readfirstlane(lds_base + uint32_t(wave * kLoadsA) * 1024u);
+  const uint32_t l_lds_b0 =
+      __builtin_amdgcn_readfirstlane(lds_base + PlanA::kStageBytes + uint32_t(wave * kLoadsB) * 1024u);
+  uint32_t l_soff_a = l_soff_a0, l_soff_b = l_soff_b0;
+  uint32_t l_slot = 0;  // byte offset of the LDS slot being filled: 0 or kStageBytes
+  int l_step = 0, l_n_steps = 1;
+  int64_t l_k = 0;
+  auto load_tile = [&](const TileState<T>& t) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      l_rsrc_a[w] = __builtin_amdgcn_readfirstlane(t.rsrc_a[w]);
+      l_rsrc_b[w] = __builtin_amdgcn_readfirstlane(t.rsrc_b[w]);
+    }
+    l_n_steps = __builtin_amdgcn_readfirstlane(t.n_steps);
+    l_step = 0;
+    l_soff_a = l_soff_a0;
+    l_soff_b = l_soff_b0;
+  };
+  auto issue_one_load = [&](int li) {  // li is a compile-time constant at every call site
+    if (li < kLoadsA)
+      plan_a.issue_one(l_rsrc_a, l_lds_a0 + l_slot, l_soff_a, li);
+    else
+      plan_b.issue_one(l_rsrc_b, l_lds_b0 + l_slot, l_soff_b, li - kLoadsA);
+  };
+  auto issue_loads = [&](auto first_tag, auto last_tag) {
+    constexpr int kFirst = decltype(first_tag)::value, kLast = decltype(last_tag)::value;
+#pragma unroll
+    for (int li = kFirst; li < kLast; ++li) issue_one_load(li);
+  };
+  auto advance_loads = [&]() {  // the stage under the cursor is fully issued: move to the next
+    l_slot ^= kStageBytes;
+    l_soff_a += plan_a.step_bytes;
+    l_soff_b += plan_b.step_bytes;
+    if (++l_step >= l_n_steps) {
+      l_k += wgs_per_xcd;
+      const int64_t id = tile_id(l_k);
+      TileState<T> t;
+      if (id >= 0) {
+        locate(id, t);
+      } else {  // nothing left: an empty descriptor
+        t.rsrc_a = make_rsrc(p.a, 0);
+        t.rsrc_b = make_rsrc(p.b, 0);
+        t.n_steps = 0x7fffffff;
+      }
+      load_tile(t);
+    }
+  };
+
+  // ---- one tile of MFMAs.  On entry the fragments of its first slice are in registers (set 0)
+  // and the loads of its second stage are partly issued; on exit the same holds for the next
+  // tile if there is one (`more`).
+  uint32_t c_slot = 0;  // byte offset of the LDS slot the MFMAs read: 0 or kStageBytes
+  auto run_tile = [&](auto atm_tag, const TileState<T>& cur, bool more, uint4 (&f0a)[TM], uint4 (&f0b)[TN]) {
     constexpr int ATM = decltype(atm_tag)::value;
     constexpr int AR = ATM > 0 ? ATM : 1;
     // The lane index as seen by this tile's address arithmetic: passed through an opaque asm so
@@ -280,100 +351,90 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    uint4 fa[2][AR], fb[2][TN];
-    auto read_set = [&](int set, int step, int kk) {
-      const unsigned char* ta = smem + (step % kStages) * kStageBytes;
-      const unsigned char* tb = ta + PlanA::kStageBytes;
+    uint4 fa[2][TM], fb[2][TN];
 #pragma unroll
-      for (int j = 0; j < TN; ++j) fb[set][j] = read_fragment<BN, B_KM>(tb, wave_j + j * 32, kk, tl);
+    for (int i = 0; i < TM; ++i) fa[0][i] = f0a[i];
 #pragma unroll
-      for (int i = 0; i < ATM; ++i) fa[set][i] = read_fragment<BM, A_KM>(ta, (2 * i + wave_row) * 32, kk, tl);
-    };
-    auto mma_set = [&](int set) {
-#pragma unroll
-      for (int i = 0; i < ATM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(fb[set][j], fa[set][i], acc[i][j]);
-    };
-    // scheduling hint: LDS reads in the shadow of the MFMAs
-    auto interleave = [&]() {
-      constexpr int kReads = (TN * (B_KM ? 2 : 1) + ATM * (A_KM ? 2 : 1));
-      constexpr int kMfma = ATM * TN;
-      if constexpr (kMfma > 0) {
-#pragma unroll
-        for (int r = 0; r < kReads; ++r) {
-          __builtin_amdgcn_sched_group_barrier(0x008, (kMfma >= 2 * kReads) ? 2 : 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-      }
-    };
-    auto prefetch_next = [&]() {
-      if (next_id >= 0) {
-        locate(next_id, next);
-        if (next.n_steps > 0) issue(next, 0);
-      }
-    };
+    for (int j = 0; j < TN; ++j) fb[0][j] = f0b[j];
 
-    const int n_steps = __builtin_amdgcn_readfirstlane(cur.n_steps);  // wave-uniform: scalar branches
-    if (n_steps > 0) {
-      // stage 0 has landed when at most the loads of stage 1 are outstanding (the stores of the
-      // previous tile's epilogue were issued between the two and are then done as well)
-      if (n_steps > 1)
-        wait_vmcnt<kLoadsPerStep>();
-      else
-        wait_vmcnt<0>();
-      __syncthreads();
-      read_set(0, 0, 0);
-      for (int step = 0; step + 1 < n_steps; ++step) {
-        read_set(1, step, 1);
-        mma_set(0);
-        interleave();
-        read_set(0, step, 2);
-        mma_set(1);
-        interleave();
-        read_set(1, step, 3);
-        mma_set(0);
-        interleave();
-        wait_vmcnt<0>();                                    // stage step+1 has landed (my part)
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // my reads of stage `step` are done
-        __syncthreads();  // stage step+1 is complete in LDS and nobody reads stage `step` any more
-        if (step + kStages < n_steps) issue(cur, step + kStages);  // refill the slot of stage `step`
-        read_set(0, step + 1, 0);
-        mma_set(1);
-        interleave();
+    // one 16-wide slice: the MFMAs of register set `set`; in their shadow the LDS reads of
+    // slice `kk_next` of stage `stage_next` into the other set (one read per two MFMAs) and
+    // the loads [L0, L1) of the stage under the load cursor (one per three MFMAs).
+    auto slice = [&](int set, bool read_next, uint32_t slot_next, int kk_next, auto l0_tag, auto l1_tag) {
+      constexpr int L0 = decltype(l0_tag)::value, L1 = decltype(l1_tag)::value;
+      const unsigned char* ta = smem + slot_next;
+      const unsigned char* tb = ta + PlanA::kStageBytes;
+      constexpr int kMfma = ATM * TN;
+      constexpr int kReads = TN + TM;  // all TM fragments are fetched: the next tile may need them
+      int reads_done = 0, loads_done = L0;
+      auto one_read = [&](int r) {
+        if (!read_next) return;
+        if (r < TN)
+          fb[set ^ 1][r] = read_fragment<BN, B_KM>(tb, wave_j + r * 32, kk_next, tl);
+        else
+          fa[set ^ 1][r - TN] = read_fragment<BM, A_KM>(ta, (2 * (r - TN) + wave_row) * 32, kk_next, tl);
+      };
+#pragma unroll
+      for (int m = 0; m < kMfma; ++m) {
+        const int i = m / TN, j = m % TN;
+        acc[i][j] = Mfma<T>::run(fb[set][j], fa[set][i], acc[i][j]);
+        if ((m & 1) && reads_done < kReads) one_read(reads_done++);
+        if (m % 3 == 2 && loads_done < L1) issue_one_load(loads_done++);
       }
-      const int last = n_steps - 1;
-      read_set(1, last, 1);
-      mma_set(0);
-      interleave();
-      read_set(0, last, 2);
-      mma_set(1);
-      interleave();
-      read_set(1, last, 3);
-      mma_set(0);
-      interleave();
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      __syncthreads();  // both stages are free: the next tile may start to arrive
-      prefetch_next();
-      mma_set(1);
-    } else {
+#pragma unroll
+      for (int r = 0; r < kReads; ++r)
+        if (r >= reads_done) one_read(r);
+#pragma unroll
+      for (int li = L0; li < L1; ++li)
+        if (li >= loads_done) issue_one_load(li);
+    };
+    using C0 = std::integral_constant<int, 0>;
+    using CE = std::integral_constant<int, kEarly>;
+    using CM = std::integral_constant<int, kMid>;
+    using CL = std::integral_constant<int, kLoads>;
+
+    const int n_steps = cur.n_steps;
+    for (int step = 0; step < n_steps; ++step) {
+      slice(0, true, c_slot, 1, CE{}, CM{});
+      slice(1, true, c_slot, 2, CM{}, CL{});
+      advance_loads();
+      slice(0, true, c_slot, 3, C0{}, C0{});
+      // everything issued so far has landed => the next stage is complete (my part); my reads
+      // of this stage are done; after the barrier that holds for the whole workgroup.  (After
+      // the last stage of the last tile this waits for empty loads and the reads below fetch
+      // fragments nobody uses: cheaper than a branch around every read.)
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       __syncthreads();
-      prefetch_next();
+      c_slot ^= kStageBytes;
+      slice(1, true, c_slot, 0, C0{}, CE{});
     }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) f0a[i] = fa[0][i];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) f0b[j] = fb[0][j];
+
     // ---- epilogue.  In the accumulators a lane owns row (lane % 32) of a sub-block and, per
     // group of four registers, four consecutive columns starting at (r/4)*8 + (lane/32)*4:
     // stored from there, a wave-wide store would touch 32 rows with 16 bytes each.  Instead a
-    // 32 x 128 sub-block is rounded, written to LDS (16-byte chunks XOR-swizzled with the row)
-    // and read back row-wise, so that every store instruction writes four full 256-byte row
-    // segments.  The scratch is the part of the second LDS stage this very wave refills
-    // afterwards, so no other wave is involved and no workgroup barrier is needed.
-    static_assert(BN == 256 && sizeof(T) == 2, "epilogue staging assumes 128 columns of 16-bit outputs per wave");
-    unsigned char* scratch[2] = {smem + kStageBytes + wave * 8192,
-                                 smem + kStageBytes + PlanA::kStageBytes + wave * 8192};
+    // 32 x 128 sub-block is rounded, written to this wave's LDS scratch (16-byte chunks
+    // XOR-swizzled with the row) and read back row-wise, so that every store instruction
+    // writes four full 256-byte row segments.
+    unsigned char* buf = smem + kStages * kStageBytes + wave * kEpilogueScratch;
+    // The output tile is written through a raw buffer descriptor (scalar base, 32-bit lane
+    // offsets): rows past the live rows of the tile fall outside the descriptor and are dropped
+    // by the bounds check; lanes past the column bound aim past the end of any descriptor.  (No
+    // lane-dependent branch: the tile bookkeeping stays provably wave-uniform around it.)
+    constexpr uint32_t kDroppedOffset = 0xffffff00u;
+    const uint32_t row_bytes_c = uint32_t(p.ldc) * 2u;
+    const int live_rows = cur.valid_i < BM ? cur.valid_i : BM;
+    const __amdgpu_buffer_rsrc_t rsrc_c =
+        __builtin_amdgcn_make_buffer_rsrc(static_cast<void*>(cur.c), 0, int(uint32_t(live_rows) * row_bytes_c), 0x00020000);
+    const int valid_j = cur.valid_j;
+    const int r = tl % 32;
+    unsigned char* wr = buf + r * 256 + (tl / 32) * 8;
+    const int rd_row = tl / 16, rd_c16 = tl % 16;  // it-th read: row = it*4 + rd_row
 #pragma unroll
     for (int i = 0; i < ATM; ++i) {
-      unsigned char* buf = scratch[i & 1];
-      const int r = tl % 32;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
 #pragma unroll
@@ -381,47 +442,61 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
           Pack4<T> out;
 #pragma unroll
           for (int e = 0; e < 4; ++e) out.v[e] = from_float<T>(acc[i][j][q * 4 + e]);
-          const int chunk = (j * 4 + q) ^ (r & 15);
-          *reinterpret_cast<Pack4<T>*>(buf + r * 256 + chunk * 16 + (tl / 32) * 8) = out;
+          *reinterpret_cast<Pack4<T>*>(wr + (((j * 4 + q) ^ (r & 15)) * 16)) = out;
         }
       }
       const int row0 = (2 * i + wave_row) * 32;
+      const int col = wave_j + rd_c16 * 8;
+      const bool col_live = col < valid_j;
 #pragma unroll
       for (int it = 0; it < 8; ++it) {
-        const int id = it * kWave + tl;
-        const int row = id / 16, c16 = id % 16;
-        const uint4 v = *reinterpret_cast<const uint4*>(buf + row * 256 + ((c16 ^ (row & 15)) * 16));
-        const int col = wave_j + c16 * 8;
-        if (row0 + row < cur.valid_i && col < cur.valid_j)
-          *reinterpret_cast<uint4*>(cur.c + int64_t(row0 + row) * p.ldc + col) = v;
+        const int row = it * 4 + rd_row;
+        const uint4 v = *reinterpret_cast<const uint4*>(buf + row * 256 + ((rd_c16 ^ (row & 15)) * 16));
+        __builtin_amdgcn_raw_buffer_store_b128(
+            __builtin_bit_cast(u32x4_t, v), rsrc_c,
+            col_live ? uint32_t(row0 + row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset, 0, 0);
       }
     }
-    // the second stage of the next tile goes out behind the stores (see the wait above)
-    if (next_id >= 0 && __builtin_amdgcn_readfirstlane(next.n_steps) > 1) issue(next, 1);
   };
 
+  // ---- prologue: first tile, its first stage in full and the head of its second
   int64_t k = blockIdx.x / kNumXcd;
   int64_t id = tile_id(k);
   if (id < 0) return;
-  TileState<T> cur, next;
+  TileState<T> cur;
   locate(id, cur);
-  if (cur.n_steps > 0) issue(cur, 0);
-  if (cur.n_steps > 1) issue(cur, 1);
+  l_k = k;
+  load_tile(cur);
+  issue_loads(std::integral_constant<int, 0>{}, std::integral_constant<int, kLoads>{});
+  advance_loads();
+  issue_loads(std::integral_constant<int, 0>{}, std::integral_constant<int, kEarly>{});
+  // stage 0 has landed once at most the kEarly younger loads are outstanding
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kEarly) : "memory");
+  __syncthreads();
+  uint4 f0a[TM], f0b[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) f0b[j] = read_fragment<BN, B_KM>(smem + PlanA::kStageBytes, wave_j + j * 32, 0, lane);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) f0a[i] = read_fragment<BM, A_KM>(smem, (2 * i + wave_row) * 32, 0, lane);
+
   while (true) {
     const int64_t next_id = tile_id(k + wgs_per_xcd);
+    const bool more = next_id >= 0;
     const int live_sub = (cur.valid_i < BM ? cur.valid_i + 31 : BM) / 32;  // live 32-row sub-blocks
     const int my_sub = __builtin_amdgcn_readfirstlane((live_sub + 1 - wave_row) / 2);  // those of this wave row
     switch (my_sub) {
-      case 0: run_tile(std::integral_constant<int, 0>{}, cur, next_id, next); break;
-      case 1: run_tile(std::integral_constant<int, 1>{}, cur, next_id, next); break;
-      case 2: run_tile(std::integral_constant<int, (TM >= 2 ? 2 : TM)>{}, cur, next_id, next); break;
-      case 3: run_tile(std::integral_constant<int, (TM >= 3 ? 3 : TM)>{}, cur, next_id, next); break;
-      default: run_tile(std::integral_constant<int, TM>{}, cur, next_id, next); break;
+      case 0: run_tile(std::integral_constant<int, 0>{}, cur, more, f0a, f0b); break;
+      case 1: run_tile(std::integral_constant<int, 1>{}, cur, more, f0a, f0b); break;
+      case 2: run_tile(std::integral_constant<int, (TM >= 2 ? 2 : TM)>{}, cur, more, f0a, f0b); break;
+      case 3: run_tile(std::integral_constant<int, (TM >= 3 ? 3 : TM)>{}, cur, more, f0a, f0b); break;
+      default: run_tile(std::integral_constant<int, TM>{}, cur, more, f0a, f0b); break;
     }
-    if (next_id < 0) break;
-    cur = next;
+    if (!more) break;
     k += wgs_per_xcd;
+    locate(next_id, cur);
   }
+  // the empty loads issued past the last stage still write (zeros) to LDS: let them finish
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 int persistent_grid() {
@@ -440,7 +515,7 @@ int persistent_grid() {
 template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD>
 int launch(const GemmArgs& p, hipStream_t s) {
   auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD>;
-  constexpr size_t smem = size_t(kStages) * (BM + BN) * kBK * 2;
+  constexpr size_t smem = size_t(kStages) * (BM + BN) * kBK * 2 + size_t(kThreads / kWave) * kEpilogueScratch;
   static bool configured = false;
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
