@@ -34,6 +34,12 @@ METRIC = "routed grouped-FFN fwd+bwd TFLOP/s + permute/unpermute GB/s, 1 MI355X"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 
+# HBM bytes per grouped-GEMM launch (fetched + written, mean over the six launches of a step),
+# from hardware counters collected in separate profiler runs of this script (FETCH_SIZE, then
+# WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB copies of
+# --traffic-probe); the summaries of those runs are kept under profiles/.  None = not measured.
+MEASURED_GEMM_TRAFFIC_BYTES = {"c2": 2.445e9, "c3": None, "c4": None}
+
 WORKLOADS = {
     "c2": dict(T=16384, H=2048, E=128, K=8, F=768, sigmoid=False, norm=True, n_group=1, topk_group=1, std=0.02),
     "c3": dict(T=16384, H=2048, E=128, K=8, F=768, sigmoid=False, norm=True, n_group=1, topk_group=1, std=0.02, zipf=1.2),
@@ -61,12 +67,13 @@ def make_inputs(cfg, seed, device):
 
 
 def cpu_baseline(cfg, seed, threads):
-    """Oracle on CPU tensors, fp32, on a bounded sample of the same workload: a quarter of
-    the tokens over all experts (the per-expert matmul loop at 1/4 of the rows per expert)."""
+    """Oracle on CPU tensors, fp32, on a bounded sample of the same workload: an eighth of
+    the tokens over all experts (the per-expert matmul loop at 1/8 of the rows per expert),
+    passes repeated until about 12 s have gone by (two or three passes)."""
     from oracle import moe_oracle as O
 
     torch.set_num_threads(threads)
-    T = cfg["T"] // 4
+    T = cfg["T"] // 8
     H, E, F, K = cfg["H"], cfg["E"], cfg["F"], cfg["K"]
     gen = torch.Generator().manual_seed(seed)
     x = (torch.randn(T, H, generator=gen) * cfg["std"]).bfloat16().float().requires_grad_(True)
@@ -86,15 +93,15 @@ def cpu_baseline(cfg, seed, threads):
         )  # fmt: skip
         out.backward(go)
         times.append(time.perf_counter() - t0)
-        if sum(times) > 25.0:
+        if sum(times) > 12.0:
             break
-    best = sorted(times)[len(times) // 2] if len(times) >= 3 else min(times)
+    best = min(times)
     return {
         "value": flops / best / 1e12,
         "unit": "TFLOP/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"{T} of {cfg['T']} tokens over all {E} experts, fp32, fwd+bwd, median of {len(times)} passes, "
+        "sample": f"{T} of {cfg['T']} tokens over all {E} experts, fp32, fwd+bwd, best of {len(times)} passes, "
         f"{best * 1e3:.0f} ms per pass",
     }
 
@@ -107,6 +114,11 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument(
+        "--traffic-probe", action="store_true",
+        help="also run three plain elementwise copies (negation) of 1 GiB before the timed region: under a counter-collecting "
+        "profiler they calibrate the HBM byte counters against a kernel of known traffic",
+    )  # fmt: skip
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the single-GPU hot path only: run it with --gpus 1 (no multi-GPU figure exists)")
@@ -143,6 +155,13 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    if args.traffic_probe:
+        src = torch.empty(1 << 28, device=dev, dtype=torch.float32).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.neg(src, out=dst)  # a plain elementwise kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     with KernelTimer() as kt:
         t0 = time.perf_counter()
         for _ in range(args.steps):
@@ -165,12 +184,12 @@ def main():
     achieved = flops_per_launch / (avg_launch_ms * 1e-3) / 1e12 if gemm_calls else 0.0
     roofline = {
         "bound": "mfma",
-        "kernel": "mfma_gemm_kernel (grouped GEMM fwd/dgrad/wgrad)",
+        "kernel": "persistent_gemm_kernel (grouped GEMM fwd / dgrad / wgrad, 256x256x64 tiles)",
         "achieved": achieved,
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_BF16_TFLOPS,
-        "traffic": None,
+        "traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(args.workload),
         "flops_per_launch": flops_per_launch,
         "avg_launch_us": avg_launch_ms * 1e3,
         "launches_per_step": gemm_calls / args.steps,

@@ -246,18 +246,40 @@ __global__ __launch_bounds__(1024) void router_finish_kernel(const float* __rest
                                                              int n_experts, int64_t n_tokens, float* __restrict__ me,
                                                              int32_t* __restrict__ hist, float* __restrict__ aux) {
   __shared__ float wave_part[1024 / kWave];
+  __shared__ float s_part[1024];
+  __shared__ int32_t n_part[1024];
+  // The block's threads form `slices` rows of `width` experts; a row sums every slices-th
+  // partial of its experts, row 0 then adds the rows up in a fixed order.
+  int width = kWave;
+  while (width < n_experts && width < 1024) width <<= 1;
+  const int slices = 1024 / width;
+  const int col = threadIdx.x % width, slice = threadIdx.x / width;
   float mine = 0.f;
-  for (int e = threadIdx.x; e < n_experts; e += 1024) {
+  for (int e0 = 0; e0 < n_experts; e0 += width) {
+    const int e = e0 + col;
     float s = 0.f;
     int32_t n = 0;
-    for (int b = 0; b < n_blocks; ++b) {
-      s += col_partial[int64_t(b) * n_experts + e];
-      n += cnt_partial[int64_t(b) * n_experts + e];
+    if (e < n_experts) {
+#pragma unroll 8
+      for (int b = slice; b < n_blocks; b += slices) {
+        s += col_partial[int64_t(b) * n_experts + e];
+        n += cnt_partial[int64_t(b) * n_experts + e];
+      }
     }
-    const float m = n_tokens > 0 ? s / float(n_tokens) : 0.f;
-    me[e] = m;
-    hist[e] = n;
-    mine += m * float(n);
+    s_part[threadIdx.x] = s;
+    n_part[threadIdx.x] = n;
+    __syncthreads();
+    if (slice == 0 && e < n_experts) {
+      for (int r = 1; r < slices; ++r) {
+        s += s_part[r * width + col];
+        n += n_part[r * width + col];
+      }
+      const float m = n_tokens > 0 ? s / float(n_tokens) : 0.f;
+      me[e] = m;
+      hist[e] = n;
+      mine += m * float(n);
+    }
+    __syncthreads();
   }
   mine = wave_sum(mine);
   if (threadIdx.x % kWave == 0) wave_part[threadIdx.x / kWave] = mine;
