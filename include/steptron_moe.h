@@ -129,6 +129,37 @@ int stm_unpermute_bwd(const void* grad_out, const void* in, const void* pos, int
                       int weight_dtype, void* grad_in, void* grad_weight, int64_t n_tokens, int top_k,
                       int64_t hidden, int64_t n_in_rows, int dtype, uint8_t* written_or_null, stm_stream_t stream);
 
+/* d input / d weight of moe_weighted_gather for ANY index, including one that names an input
+ * row from several slots (the reference accumulates them with index_add_, moe_utils.py:302-305;
+ * its own test uses such an index, tests/test_moe_utils.py:61-101).  Contributions to a row are
+ * added in fp32 in ascending flat-slot order (deterministic) and rounded once; rows nobody
+ * names are zero.  Workspace: stm_unpermute_bwd_general_workspace_bytes(T*K, n_in_rows). */
+size_t stm_unpermute_bwd_general_workspace_bytes(int64_t n_slots, int64_t n_in_rows);
+int stm_unpermute_bwd_general(const void* grad_out, const void* in, const void* pos, int pos_is_i64, const void* weight,
+                              int weight_dtype, void* grad_in, void* grad_weight, int64_t n_tokens, int top_k,
+                              int64_t hidden, int64_t n_in_rows, int dtype, void* workspace, size_t workspace_bytes,
+                              stm_stream_t stream);
+
+/* Building blocks of the TE-style permutation helpers (reference
+ * steptronoss/model/utils/permute_utils.py:43-277).
+ * stm_sort_by_key: stable sort of the entries with 0 <= key < key_bound (others are dropped):
+ *   sorted_key int32 [n] ascending, padded with INT32_MAX; sorted_index int32 [n] the entries'
+ *   flat positions; n_valid_out (device int32, optional) the number kept.  key_bound <= 2^24.
+ *   This is the argsort of permute_utils.py:109-113 and the transposed nonzero of :63.
+ * stm_gather_rows: out[j] = idx[j] in [0, n_src_rows) ? x[idx[j]] : 0  (:32-41).
+ * stm_segment_sum_rows: out[r] = sum over list entries j with sorted_key[j] == r of
+ *   weight[i_j] * src[i_j / src_div], i_j = sorted_index[j]; fp32 sums in list order, rounded
+ *   once; the deterministic form of the scatter_add_ of :201,:232. */
+size_t stm_sort_by_key_workspace_bytes(int64_t n, int64_t key_bound);
+int stm_sort_by_key(const void* keys, int keys_are_i64, int64_t n, int64_t key_bound, int32_t* sorted_key,
+                    int32_t* sorted_index, int32_t* n_valid_out, void* workspace, size_t workspace_bytes,
+                    stm_stream_t stream);
+int stm_gather_rows(const void* x, const void* idx, int idx_is_i64, void* out, int64_t n_out_rows, int64_t row_bytes,
+                    int64_t n_src_rows, stm_stream_t stream);
+int stm_segment_sum_rows(const void* src, const int32_t* sorted_key, const int32_t* sorted_index, int64_t n_sorted,
+                         int64_t src_div, const void* weight_or_null, int weight_dtype, void* out, int64_t n_out_rows,
+                         int64_t hidden, int dtype, stm_stream_t stream);
+
 /* Inspects a position map: status[STM_ST_N_VALID] = number of non-negative entries,
  * status[STM_ST_MAX_ROW_PLUS1] = 1 + largest entry, status[STM_ST_NOT_INJECTIVE] set when
  * two non-negative entries are equal, status[STM_ST_ROW_OUT_OF_RANGE] when one is

@@ -46,6 +46,12 @@ SIGNATURES = {
     "stm_permute_bwd": (I, [P, P, I, P, L, I, L, L, I, P]),
     "stm_unpermute_fwd": (I, [P, P, I, P, I, P, L, I, L, L, I, P]),
     "stm_unpermute_bwd": (I, [P, P, P, I, P, I, P, P, L, I, L, L, I, P, P]),
+    "stm_unpermute_bwd_general_workspace_bytes": (Z, [L, L]),
+    "stm_unpermute_bwd_general": (I, [P, P, P, I, P, I, P, P, L, I, L, L, I, P, Z, P]),
+    "stm_sort_by_key_workspace_bytes": (Z, [L, L]),
+    "stm_sort_by_key": (I, [P, I, L, L, P, P, P, P, Z, P]),
+    "stm_gather_rows": (I, [P, P, I, P, L, L, L, P]),
+    "stm_segment_sum_rows": (I, [P, P, P, L, L, P, I, P, L, L, I, P]),
     "stm_index_check": (I, [P, I, L, L, P, P, P]),
     "stm_gemm_workspace_bytes": (Z, [L, I]),
     "stm_grouped_gemm": (I, [P, P, P, P, I, L, I, I, I, I, P, Z, P]),

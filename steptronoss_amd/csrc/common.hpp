@@ -122,4 +122,11 @@ inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintp
 
 inline size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// Stable sort of the valid slots of a position map by the row they name (routing.hip); used
+// by the combine backward when several slots name one row.
+size_t sort_by_row_workspace_bytes(int64_t n_slots, int64_t n_rows);
+int sort_slots_by_row(const void* pos, int pos_is_i64, int64_t n_slots, int64_t n_rows, int32_t* sorted_row,
+                      int32_t* sorted_slot, int32_t* n_valid_out, void* workspace, size_t workspace_bytes,
+                      hipStream_t stream);
+
 }  // namespace stm

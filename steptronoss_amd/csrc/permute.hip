@@ -212,6 +212,57 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_bwd_kernel(
   }
 }
 
+// ---------------------------------------------------------------- sums over sorted segments
+// out[r] = sum over the entries j of the sorted list with sorted_key[j] == r of
+// weight[slot_j] * src[slot_j / src_div] (slot_j = sorted_slot[j]; weight 1 when absent), each
+// product rounded to T like a stored row, added in fp32 in list order, rounded once; rows
+// without entries become zero.  One workgroup per output row.  With src = d out, src_div =
+// top_k this is d rows of the combine for a position map that names rows several times; with
+// src_div = 1 it is a weighted scatter-add of rows made deterministic.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kRowThreads) void segment_sum_rows_kernel(
+    const T* __restrict__ src, const int32_t* __restrict__ sorted_key, const int32_t* __restrict__ sorted_slot,
+    int64_t n_sorted, int64_t src_div, const void* __restrict__ weight, int wdtype, T* __restrict__ out, int64_t hidden) {
+  using P = Pack<T, VEC>;
+  const int64_t r = blockIdx.x;
+  int64_t lo = 0, hi = n_sorted;
+  while (lo < hi) {  // first entry with sorted_key >= r
+    const int64_t mid = (lo + hi) / 2;
+    if (sorted_key[mid] < r) lo = mid + 1; else hi = mid;
+  }
+  const int64_t units = hidden / VEC;
+  for (int64_t u = threadIdx.x; u < units; u += kRowThreads) {
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+    for (int64_t i = lo; i < n_sorted && sorted_key[i] == r; ++i) {
+      const int64_t slot = sorted_slot[i];
+      const float w = weight ? round_through<T>(load_weight_any(weight, wdtype, slot)) : 1.f;
+      const P g = reinterpret_cast<const P*>(src + (slot / src_div) * hidden)[u];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] += round_through<T>(to_float(g.v[j]) * w);
+    }
+    P o;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) o.v[j] = from_float<T>(acc[j]);
+    reinterpret_cast<P*>(out + r * hidden)[u] = o;
+  }
+}
+
+// ---------------------------------------------------------------- row gather
+// out[j] = idx[j] in [0, n_src) ? x[idx[j]] : 0; one wavefront per output row.
+template <typename V, bool I64>
+__global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const V* __restrict__ x, const void* __restrict__ idx,
+                                                                  V* __restrict__ out, int64_t n_out, int64_t units,
+                                                                  int64_t n_src) {
+  const int64_t j = int64_t(blockIdx.x) * (kRowThreads / kWave) + threadIdx.x / kWave;
+  if (j >= n_out) return;
+  const int64_t i = load_pos<I64>(idx, j);
+  const bool ok = i >= 0 && i < n_src;
+  V zero{};
+  for (int64_t u = threadIdx.x % kWave; u < units; u += kWave) out[j * units + u] = ok ? x[i * units + u] : zero;
+}
+
 // ---------------------------------------------------------------- index check
 template <bool I64>
 __global__ void claim_rows_kernel(const void* __restrict__ pos, int64_t n_slots, int64_t n_rows,
@@ -369,6 +420,46 @@ int dispatch_unpermute_bwd(const void* go, const void* in, const void* pos, int 
   return launch_status();
 }
 
+template <typename T>
+int dispatch_segment_sum_rows(const void* src, const int32_t* sorted_key, const int32_t* sorted_slot, int64_t n_sorted,
+                              int64_t src_div, const void* w, int wdtype, void* out, int64_t hidden, int64_t n_rows,
+                              hipStream_t s) {
+  const T* g = static_cast<const T*>(src);
+  T* o = static_cast<T*>(out);
+  const unsigned grid = unsigned(n_rows);
+  if (can_vectorise<T>(hidden, {src, out, out}))
+    segment_sum_rows_kernel<T, wide_vec<T>()><<<grid, kRowThreads, 0, s>>>(g, sorted_key, sorted_slot, n_sorted, src_div, w,
+                                                                          wdtype, o, hidden);
+  else
+    segment_sum_rows_kernel<T, 1><<<grid, kRowThreads, 0, s>>>(g, sorted_key, sorted_slot, n_sorted, src_div, w, wdtype, o,
+                                                               hidden);
+  return launch_status();
+}
+
+int segment_sum_rows_any(const void* src, const int32_t* sorted_key, const int32_t* sorted_slot, int64_t n_sorted,
+                         int64_t src_div, const void* w, int wdtype, void* out, int64_t hidden, int64_t n_rows, int dtype,
+                         hipStream_t s) {
+  switch (dtype) {
+    case STM_F32: return dispatch_segment_sum_rows<float>(src, sorted_key, sorted_slot, n_sorted, src_div, w, wdtype, out, hidden, n_rows, s);
+    case STM_F16: return dispatch_segment_sum_rows<f16_t>(src, sorted_key, sorted_slot, n_sorted, src_div, w, wdtype, out, hidden, n_rows, s);
+    case STM_BF16: return dispatch_segment_sum_rows<bf16_t>(src, sorted_key, sorted_slot, n_sorted, src_div, w, wdtype, out, hidden, n_rows, s);
+    default: return STM_ERR_UNSUPPORTED;
+  }
+}
+
+template <typename V>
+int launch_gather_rows(const void* x, const void* idx, int idx_is_i64, void* out, int64_t n_out, int64_t row_bytes,
+                       int64_t n_src, hipStream_t s) {
+  const int rows_per_block = kRowThreads / kWave;
+  const unsigned grid = unsigned((n_out + rows_per_block - 1) / rows_per_block);
+  const int64_t units = row_bytes / int64_t(sizeof(V));
+  if (idx_is_i64)
+    gather_rows_kernel<V, true><<<grid, kRowThreads, 0, s>>>(static_cast<const V*>(x), idx, static_cast<V*>(out), n_out, units, n_src);
+  else
+    gather_rows_kernel<V, false><<<grid, kRowThreads, 0, s>>>(static_cast<const V*>(x), idx, static_cast<V*>(out), n_out, units, n_src);
+  return launch_status();
+}
+
 inline bool bad_rows(int64_t n_tokens, int top_k, int64_t width) {
   return n_tokens < 0 || top_k < 0 || width < 0 || n_tokens > 0x7fffffffll;
 }
@@ -459,6 +550,82 @@ int stm_unpermute_bwd(const void* grad_out, const void* in, const void* pos, int
     case STM_F16: return dispatch_unpermute_bwd<f16_t>(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k, hidden, n_in_rows, written_or_null, s);
     case STM_BF16: return dispatch_unpermute_bwd<bf16_t>(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k, hidden, n_in_rows, written_or_null, s);
     default: return STM_ERR_UNSUPPORTED;
+  }
+}
+
+size_t stm_unpermute_bwd_general_workspace_bytes(int64_t n_slots, int64_t n_in_rows) {
+  if (n_slots < 0 || n_in_rows < 0) return 0;
+  return 2 * stm::round_up(size_t(n_slots) * sizeof(int32_t), 256) + stm::sort_by_row_workspace_bytes(n_slots, n_in_rows);
+}
+
+int stm_unpermute_bwd_general(const void* grad_out, const void* in, const void* pos, int pos_is_i64, const void* weight,
+                              int weight_dtype, void* grad_in, void* grad_weight, int64_t n_tokens, int top_k,
+                              int64_t hidden, int64_t n_in_rows, int dtype, void* workspace, size_t workspace_bytes,
+                              stm_stream_t stream) {
+  using namespace stm;
+  if (bad_rows(n_tokens, top_k, hidden) || n_in_rows < 0) return STM_ERR_ARG;
+  if (n_in_rows > 0x7fffffffll) return STM_ERR_UNSUPPORTED;
+  const int64_t n_slots = n_tokens * top_k;
+  if (n_slots > 0 && workspace_bytes < stm_unpermute_bwd_general_workspace_bytes(n_slots, n_in_rows))
+    return STM_ERR_WORKSPACE;
+  // d weight (and a first, possibly clashing, version of d rows) as for an injective map
+  int st = stm_unpermute_bwd(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k,
+                             hidden, n_in_rows, dtype, nullptr, stream);
+  if (st != STM_OK || n_in_rows == 0 || hidden == 0) return st;
+  if (!grad_in) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  unsigned char* w = static_cast<unsigned char*>(workspace);
+  const size_t list_bytes = round_up(size_t(n_slots) * sizeof(int32_t), 256);
+  int32_t* sorted_row = reinterpret_cast<int32_t*>(w);
+  int32_t* sorted_slot = reinterpret_cast<int32_t*>(w + list_bytes);
+  if (n_slots > 0) {
+    if (!workspace) return STM_ERR_WORKSPACE;
+    st = sort_slots_by_row(pos, pos_is_i64, n_slots, n_in_rows, sorted_row, sorted_slot, nullptr, w + 2 * list_bytes,
+                           workspace_bytes - 2 * list_bytes, s);
+    if (st != STM_OK) return st;
+  }
+  return segment_sum_rows_any(grad_out, sorted_row, sorted_slot, n_slots, top_k, weight, weight_dtype, grad_in, hidden,
+                              n_in_rows, dtype, s);
+}
+
+size_t stm_sort_by_key_workspace_bytes(int64_t n, int64_t key_bound) {
+  if (n < 0 || key_bound < 0) return 0;
+  return stm::sort_by_row_workspace_bytes(n, key_bound);
+}
+
+int stm_sort_by_key(const void* keys, int keys_are_i64, int64_t n, int64_t key_bound, int32_t* sorted_key,
+                    int32_t* sorted_index, int32_t* n_valid_out, void* workspace, size_t workspace_bytes,
+                    stm_stream_t stream) {
+  return stm::sort_slots_by_row(keys, keys_are_i64, n, key_bound, sorted_key, sorted_index, n_valid_out, workspace,
+                                workspace_bytes, stm::as_stream(stream));
+}
+
+int stm_segment_sum_rows(const void* src, const int32_t* sorted_key, const int32_t* sorted_index, int64_t n_sorted,
+                         int64_t src_div, const void* weight_or_null, int weight_dtype, void* out, int64_t n_out_rows,
+                         int64_t hidden, int dtype, stm_stream_t stream) {
+  using namespace stm;
+  if (n_sorted < 0 || n_out_rows < 0 || hidden < 0 || src_div < 1 || n_out_rows > 0x7fffffffll) return STM_ERR_ARG;
+  if (weight_or_null && (weight_dtype < STM_F32 || weight_dtype > STM_BF16)) return STM_ERR_UNSUPPORTED;
+  if (n_out_rows == 0 || hidden == 0) return STM_OK;
+  if (!out || (n_sorted > 0 && (!src || !sorted_key || !sorted_index))) return STM_ERR_ARG;
+  return segment_sum_rows_any(src, sorted_key, sorted_index, n_sorted, src_div, weight_or_null, weight_dtype, out, hidden,
+                              n_out_rows, dtype, as_stream(stream));
+}
+
+int stm_gather_rows(const void* x, const void* idx, int idx_is_i64, void* out, int64_t n_out_rows, int64_t row_bytes,
+                    int64_t n_src_rows, stm_stream_t stream) {
+  using namespace stm;
+  if (n_out_rows < 0 || row_bytes < 0 || n_src_rows < 0) return STM_ERR_ARG;
+  if (n_out_rows == 0 || row_bytes == 0) return STM_OK;
+  if (!idx || !out || (n_src_rows > 0 && !x)) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  const void* xa = x ? x : out;
+  switch (copy_unit_bytes(row_bytes, xa, out)) {
+    case 16: return launch_gather_rows<uint4>(x, idx, idx_is_i64, out, n_out_rows, row_bytes, n_src_rows, s);
+    case 8: return launch_gather_rows<uint2>(x, idx, idx_is_i64, out, n_out_rows, row_bytes, n_src_rows, s);
+    case 4: return launch_gather_rows<uint32_t>(x, idx, idx_is_i64, out, n_out_rows, row_bytes, n_src_rows, s);
+    case 2: return launch_gather_rows<uint16_t>(x, idx, idx_is_i64, out, n_out_rows, row_bytes, n_src_rows, s);
+    default: return launch_gather_rows<uint8_t>(x, idx, idx_is_i64, out, n_out_rows, row_bytes, n_src_rows, s);
   }
 }
 

@@ -257,7 +257,102 @@ int run_sort(const void* ids, int ids_are_i64, int64_t n_slots, int n_experts, c
   return launch_status();
 }
 
+// ---------------------------------------------------------------- slots sorted by row
+// Helpers of the two-pass (12 bits each) least-significant-digit radix sort below.
+__global__ void copy_i32_kernel(int32_t* dst, const int32_t* src, int64_t n) {
+  const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
+template <bool I64>
+__global__ void row_digit_kernel(const void* __restrict__ keys, int64_t n, int64_t n_rows, int shift,
+                                 int32_t* __restrict__ digit) {
+  const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int64_t k = I64 ? static_cast<const int64_t*>(keys)[i] : int64_t(static_cast<const int32_t*>(keys)[i]);
+  digit[i] = (k < 0 || k >= n_rows) ? -1 : int32_t((k >> shift) & (kMaxExperts - 1));
+}
+
+template <bool I64>
+__global__ void scatter_pairs_kernel(const int32_t* __restrict__ dest, const void* __restrict__ keys,
+                                     const int32_t* __restrict__ vals_or_null, int64_t n,
+                                     int32_t* __restrict__ keys_out, int32_t* __restrict__ vals_out) {
+  const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int32_t d = dest[i];
+  if (d < 0) return;
+  keys_out[d] = I64 ? int32_t(static_cast<const int64_t*>(keys)[i]) : static_cast<const int32_t*>(keys)[i];
+  vals_out[d] = vals_or_null ? vals_or_null[i] : int32_t(i);
+}
+
 }  // namespace
+
+namespace {
+inline size_t slots_bytes(int64_t n_slots) { return round_up(size_t(n_slots) * sizeof(int32_t), 256); }
+inline int digits_of(int64_t n_rows) { return int(n_rows < kMaxExperts ? n_rows : kMaxExperts); }
+}  // namespace
+
+size_t sort_by_row_workspace_bytes(int64_t n_slots, int64_t n_rows) {
+  // digit, dest, keys1, vals1, then the counter rows of the counting sort, then status words
+  return 4 * slots_bytes(n_slots) + stm_route_workspace_bytes(n_slots, digits_of(n_rows)) + 256;
+}
+
+// The valid slots of a position map (0 <= pos < n_rows), stably sorted by the row they name:
+// sorted_row[j] ascending (padded with INT32_MAX up to n_slots), sorted_slot[j] the flat slot;
+// n_valid_out (optional, device) receives the number of valid slots.
+// Every pass is the stable counting sort of the routing kernels on one 12-bit digit.
+int sort_slots_by_row(const void* pos, int pos_is_i64, int64_t n_slots, int64_t n_rows, int32_t* sorted_row,
+                      int32_t* sorted_slot, int32_t* n_valid_out, void* workspace, size_t workspace_bytes,
+                      hipStream_t stream) {
+  if (n_slots < 0 || n_rows < 0) return STM_ERR_ARG;
+  if (n_rows > (int64_t(1) << 24) || n_slots > (int64_t(1) << 31) - 1) return STM_ERR_UNSUPPORTED;
+  if (n_slots == 0 || n_rows == 0) {
+    if (n_valid_out) fill_i32_kernel<<<1, 64, 0, stream>>>(n_valid_out, 1, 0);
+    if (n_slots && sorted_row)
+      fill_i32_kernel<<<unsigned((n_slots + 255) / 256), 256, 0, stream>>>(sorted_row, n_slots, 0x7fffffff);
+    return launch_status();
+  }
+  if (!pos || !sorted_row || !sorted_slot || !workspace) return STM_ERR_ARG;
+  if (workspace_bytes < sort_by_row_workspace_bytes(n_slots, n_rows)) return STM_ERR_WORKSPACE;
+  unsigned char* w = static_cast<unsigned char*>(workspace);
+  int32_t* digit = reinterpret_cast<int32_t*>(w);
+  int32_t* dest = reinterpret_cast<int32_t*>(w + slots_bytes(n_slots));
+  int32_t* keys1 = reinterpret_cast<int32_t*>(w + 2 * slots_bytes(n_slots));
+  int32_t* vals1 = reinterpret_cast<int32_t*>(w + 3 * slots_bytes(n_slots));
+  void* counters = w + 4 * slots_bytes(n_slots);
+  const size_t counters_bytes = stm_route_workspace_bytes(n_slots, digits_of(n_rows));
+  int32_t* status = reinterpret_cast<int32_t*>(w + 4 * slots_bytes(n_slots) + counters_bytes);
+  const unsigned grid = unsigned((n_slots + 255) / 256);
+  const bool two_passes = n_rows > kMaxExperts;
+  fill_i32_kernel<<<1, 64, 0, stream>>>(status, STM_STATUS_WORDS, 0);
+  fill_i32_kernel<<<grid, 256, 0, stream>>>(sorted_row, n_slots, 0x7fffffff);
+  int32_t* keys_a = two_passes ? keys1 : sorted_row;
+  int32_t* vals_a = two_passes ? vals1 : sorted_slot;
+  if (two_passes) fill_i32_kernel<<<grid, 256, 0, stream>>>(keys1, n_slots, -1);
+  // pass on the low digit
+  if (pos_is_i64)
+    row_digit_kernel<true><<<grid, 256, 0, stream>>>(pos, n_slots, n_rows, 0, digit);
+  else
+    row_digit_kernel<false><<<grid, 256, 0, stream>>>(pos, n_slots, n_rows, 0, digit);
+  int st = run_sort(digit, 0, n_slots, digits_of(n_rows), nullptr, 0, nullptr, nullptr, dest, status, counters,
+                    counters_bytes, stream);
+  if (st != STM_OK) return st;
+  if (n_valid_out) copy_i32_kernel<<<1, 64, 0, stream>>>(n_valid_out, status + STM_ST_N_VALID, 1);
+  if (pos_is_i64)
+    scatter_pairs_kernel<true><<<grid, 256, 0, stream>>>(dest, pos, nullptr, n_slots, keys_a, vals_a);
+  else
+    scatter_pairs_kernel<false><<<grid, 256, 0, stream>>>(dest, pos, nullptr, n_slots, keys_a, vals_a);
+  if (two_passes) {  // pass on the high digit (the tail of keys1 is -1: dropped)
+    const int high_digits = int(((n_rows - 1) >> 12) + 1);
+    row_digit_kernel<false><<<grid, 256, 0, stream>>>(keys1, n_slots, n_rows, 12, digit);
+    st = run_sort(digit, 0, n_slots, high_digits, nullptr, 0, nullptr, nullptr, dest, status, counters, counters_bytes,
+                  stream);
+    if (st != STM_OK) return st;
+    scatter_pairs_kernel<false><<<grid, 256, 0, stream>>>(dest, keys1, vals1, n_slots, sorted_row, sorted_slot);
+  }
+  return launch_status();
+}
+
 }  // namespace stm
 
 extern "C" {

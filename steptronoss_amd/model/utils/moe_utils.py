@@ -38,7 +38,9 @@ class Settings:
     validate: the stand-alone ``histogram`` / ``index_compute`` read the device status
         words back (one small host sync, as the reference's own checks do) and raise the
         reference's errors.  ``routed_grouped_ffn`` never synchronises unless
-        ``validate_fused`` is set.
+        ``validate_fused`` is set; with it the op also reproduces the reference's early-out
+        for a batch in which no slot is routed (``x * token_weights.sum()``), which needs the
+        routed count on the host.
     """
 
     validate: bool = True
@@ -289,12 +291,20 @@ class _MoEWeightedGather(torch.autograd.Function):
             st = _check_index(pos, n_rows)
             if st[_lib.ST_ROW_OUT_OF_RANGE]:
                 raise IndexError("index out of range in moe_weighted_gather")
-            if st[_lib.ST_NOT_INJECTIVE]:
-                raise NotImplementedError(
-                    "hip_gfx950 moe_weighted_gather backward: several slots name the same input row; "
-                    "only position maps produced by index_compute (injective) are supported"
-                )
             grad_in = torch.empty_like(inp)
+            if st[_lib.ST_NOT_INJECTIVE]:
+                # several slots name one input row (never the case for index_compute's maps):
+                # slots sorted by row, one deterministic fp32 sum per row
+                n_tokens, top_k = pos.shape
+                gw = torch.empty_like(w)
+                nbytes = _lib.load().stm_unpermute_bwd_general_workspace_bytes(pos.numel(), n_rows)
+                ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+                call(
+                    "stm_unpermute_bwd_general", ptr(go), ptr(inp), ptr(pos), is_i64(pos), ptr(w), dtype_code(w.dtype),
+                    ptr(grad_in), ptr(gw), n_tokens, top_k, inp.shape[1], n_rows, dtype_code(inp.dtype), ptr(ws), nbytes,
+                    stream(),
+                )  # fmt: skip
+                return grad_in, None, gw
             covers_all = st[_lib.ST_N_VALID] == n_rows
             written = None if covers_all else torch.zeros((n_rows,), device=dev, dtype=torch.uint8)
             gw = _combine_rows_bwd(go, inp, pos, w, grad_in, written)
@@ -622,6 +632,11 @@ def hip_routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights):
     ids = token_expert_ids.contiguous()
     tw = token_weights.contiguous()
     with torch.cuda.device(dev):
+        if settings.validate_fused and not bool((ids >= 0).any()):
+            # The reference reads the routed count back on the host and, when it is zero, returns
+            # x * sum(weights) (moe_utils.py:230-232).  Only the validating mode pays for that
+            # read-back; without it an all-unrouted batch gives zeros (nothing to combine).
+            return x * token_weights.sum()
         fused, limit = _swiglu_limit_of(act, w1.shape[1], x.dtype, dev)
         if fused:
             return _FusedRoutedFFN.apply(w1c, w2c, xc, ids, tw, limit)

@@ -247,3 +247,27 @@ def test_layer_matches_oracle_on_reduced_configs(name, T, E, tol):
     }
     worst = max(errs.values())
     assert worst <= tol, errs
+
+
+def test_nothing_routed_early_out_matches_reference_when_validating():
+    # reference moe_utils.py:230-232: with no routed slot at all the op returns x * sum(weights)
+    from steptronoss_amd.model.common.feed_forward import swiglu
+    from steptronoss_amd.model.utils import moe_utils as M
+
+    gen = torch.Generator().manual_seed(3)
+    T, H, E, K, F = 12, 32, 4, 2, 16
+    x = torch.randn(T, H, generator=gen).to(DEV)
+    w1 = torch.randn(E, 2 * F, H, generator=gen).to(DEV)
+    w2 = torch.randn(E, H, F, generator=gen).to(DEV)
+    ids = torch.full((T, K), -1, dtype=torch.int64, device=DEV)
+    tw = torch.rand(T, K, generator=gen).to(DEV)
+    old = M.settings.validate_fused
+    try:
+        M.settings.validate_fused = True
+        out = M.routed_grouped_ffn(w1, w2, swiglu, x, ids, tw)
+        assert torch.allclose(out, x * tw.sum())
+        M.settings.validate_fused = False
+        out = M.routed_grouped_ffn(w1, w2, swiglu, x, ids, tw)
+        assert float(out.abs().sum()) == 0.0  # no read-back: nothing to combine
+    finally:
+        M.settings.validate_fused = old

@@ -228,12 +228,57 @@ def test_combine_backward_zeroes_unnamed_rows():
     assert torch.allclose(rows.grad[3], w[0, 1].detach().expand(16))
 
 
-def test_combine_backward_rejects_shared_rows_loudly():
-    rows = torch.randn(3, 8, device=DEV, requires_grad=True)
-    w = torch.rand(2, 2, device=DEV, requires_grad=True)
-    out = M.moe_weighted_gather(rows, torch.tensor([[2, 0], [1, 2]], device=DEV), w)
-    with pytest.raises(NotImplementedError):
-        out.sum().backward()
+def test_combine_backward_reference_kat_shared_rows():
+    # reference tests/test_moe_utils.py:81-92: row 2 is named by two slots
+    x = torch.tensor([[1.0, 2.0], [3.0, 4.0], [5.0, 6.0]], device=DEV, requires_grad=True)
+    idx = torch.tensor([[2, 0], [1, 2]], dtype=torch.int64, device=DEV)
+    w = torch.tensor([[0.2, 0.8], [1.0, 0.5]], device=DEV, requires_grad=True)
+    M.moe_weighted_gather(x, idx, w).sum().backward()
+    assert torch.allclose(x.grad.cpu(), torch.tensor([[0.8, 0.8], [1.0, 1.0], [0.7, 0.7]]))
+    assert torch.allclose(w.grad.cpu(), torch.tensor([[11.0, 3.0], [7.0, 11.0]]))
+
+
+def test_combine_backward_reference_kat_negative_indices():
+    # reference tests/test_moe_utils.py:95-104
+    x = torch.tensor([[1.0, 2.0], [3.0, 4.0], [5.0, 6.0]], device=DEV, requires_grad=True)
+    idx = torch.tensor([[2, -1], [1, -2]], dtype=torch.int64, device=DEV)
+    w = torch.tensor([[0.2, 0.8], [1.0, 0.5]], device=DEV, requires_grad=True)
+    M.moe_weighted_gather(x, idx, w).sum().backward()
+    assert torch.allclose(x.grad.cpu(), torch.tensor([[0.0, 0.0], [1.0, 1.0], [0.2, 0.2]]))
+    assert torch.allclose(w.grad.cpu(), torch.tensor([[11.0, 0.0], [7.0, 0.0]]))
+
+
+@pytest.mark.parametrize(
+    "T,K,H,n_rows,dtype,idt",
+    [
+        (300, 4, 64, 97, torch.float32, torch.int64),  # many slots per row, one sort pass
+        (700, 3, 72, 5000, torch.bfloat16, torch.int32),  # > 4096 rows: two sort passes, some rows unnamed
+        (64, 8, 40, 9000, torch.float16, torch.int64),  # mostly unnamed rows, odd width
+    ],
+)
+def test_combine_backward_any_index_matches_oracle(T, K, H, n_rows, dtype, idt):
+    gen = torch.Generator().manual_seed(11)
+    pos = torch.randint(-n_rows // 8, n_rows, (T, K), generator=gen).to(idt)  # repeats and negatives
+    rows = torch.randn(n_rows, H, generator=gen).to(dtype)
+    w = torch.rand(T, K, generator=gen)
+    go = torch.randn(T, H, generator=gen).to(dtype)
+    rr = rows.clone().float().requires_grad_(True)
+    wr = w.clone().requires_grad_(True)
+    O.moe_weighted_gather(rr, pos, wr).backward(go.float())
+    rg = rows.to(DEV).requires_grad_(True)
+    wg = w.to(DEV).requires_grad_(True)
+    out = M.moe_weighted_gather(rg, pos.to(DEV), wg)
+    out.backward(go.to(DEV))
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    assert rel_l2(rg.grad, rr.grad) <= tol
+    assert rel_l2(wg.grad, wr.grad) <= tol
+    unnamed = torch.ones(n_rows, dtype=torch.bool)
+    unnamed[pos[pos >= 0].long()] = False
+    assert float(rg.grad.cpu()[unnamed].abs().sum()) == 0.0
+    # deterministic: a second run gives the same bits
+    rg2 = rows.to(DEV).requires_grad_(True)
+    M.moe_weighted_gather(rg2, pos.to(DEV), wg.detach().requires_grad_(True)).backward(go.to(DEV))
+    assert torch.equal(rg.grad, rg2.grad)
 
 
 def test_cpu_tensors_are_refused():
