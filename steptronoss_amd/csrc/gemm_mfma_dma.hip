@@ -33,6 +33,7 @@
 //            the four rows a transposing read touches land in the four quarters of the banks.
 // A wave-wide buffer_load ... lds writes 1024 consecutive LDS bytes (lane l at +16*l), so the
 // swizzle is applied on the global-address side.
+#include <cstdlib>
 #include <type_traits>
 
 #include "gemm_common.hpp"
@@ -67,8 +68,7 @@ struct Mfma<f16_t> {
 
 constexpr int kBK = 64;  // contraction elements per stage
 constexpr int kStages = 2;
-constexpr int kThreads = 256;
-constexpr int kEpilogueScratch = 8192;  // bytes per wave, behind the stages
+constexpr int kEpilogueBytes = 32768;  // output staging of all waves, behind the stages
 
 template <typename T>
 struct alignas(sizeof(T) * 4) Pack4 {
@@ -101,10 +101,10 @@ __device__ __forceinline__ void dma16(i32x4_t rsrc, uint32_t lds_addr, uint32_t 
 // lane inside "its" load depends on the load index only through its parity (via the swizzle),
 // so two VGPRs per operand describe all of them; the first row of the load goes into the
 // scalar offset.
-template <int R, bool KM>
+template <int R, bool KM, int WAVES>
 struct OperandPlan {
   static constexpr int kStageBytes = R * kBK * 2;  // 16-bit elements
-  static constexpr int kLoadsPerWave = kStageBytes / 1024 / (kThreads / kWave);
+  static constexpr int kLoadsPerWave = kStageBytes / 1024 / WAVES;
   static constexpr int kRowsPerLoad = KM ? 1024 / (R * 2) : 8;  // stored rows covered by one load
   static_assert(kLoadsPerWave % 2 == 0, "the parity trick needs an even number of loads per wave");
   static_assert(!KM || kRowsPerLoad == 2 || kRowsPerLoad == 4, "KM tiles of 128 or 256 columns");
@@ -180,11 +180,18 @@ struct TileState {
   int valid_i, valid_j, n_steps;
 };
 
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD>
-__global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
-  constexpr int TM = BM / 64, TN = BN / 64;  // 32x32 MFMA tiles per wave (waves are laid out 2 x 2)
-  using PlanA = OperandPlan<BM, A_KM>;
-  using PlanB = OperandPlan<BN, B_KM>;
+// WAVES = 4: one wave per SIMD, 2 x 2 waves of 128 x 128 outputs each.
+// WAVES = 8: two waves per SIMD, 4 x 2 waves of 64 x 128 outputs each: while one wave of a SIMD
+//            sits in the issue of a load, the other one keeps the MFMA pipe busy.
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES>
+__global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs p) {
+  constexpr int WROWS = WAVES / 2;                   // wave rows; two wave columns
+  constexpr int TM = BM / 32 / WROWS, TN = BN / 64;  // 32x32 MFMA tiles per wave
+  constexpr int kEpilogueScratch = kEpilogueBytes / WAVES;  // per wave: 32 rows x kStageCols outputs
+  constexpr int kStageCols = kEpilogueScratch / 32 / 2;     // 128 (4 waves) or 64 (8 waves)
+  constexpr int kColRounds = (BN / 2) / kStageCols;
+  using PlanA = OperandPlan<BM, A_KM, WAVES>;
+  using PlanB = OperandPlan<BN, B_KM, WAVES>;
   constexpr uint32_t kStageBytes = PlanA::kStageBytes + PlanB::kStageBytes;
   constexpr int kLoadsA = PlanA::kLoadsPerWave, kLoadsB = PlanB::kLoadsPerWave;
   constexpr int kLoads = kLoadsA + kLoadsB;  // per wave per stage
@@ -193,7 +200,8 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
   // of step g+1; they have landed when step g+1 reaches its third quarter.
   constexpr int kEarly = kLoads * 3 / 8;
   constexpr int kMid = kEarly + (kLoads - kEarly + 1) / 2;
-  static_assert(BN == 256 && sizeof(T) == 2, "epilogue staging assumes 128 columns of 16-bit outputs per wave");
+  static_assert(BN == 256 && sizeof(T) == 2 && (kStageCols == 128 || kStageCols == 64),
+                "epilogue staging assumes 128 columns of 16-bit outputs per wave, staged 128 or 64 at a time");
   extern __shared__ __align__(1024) unsigned char smem[];
 
   // ---- this workgroup's tiles: XCD x = blockIdx % 8 owns tiles [x*per_xcd, (x+1)*per_xcd);
@@ -270,9 +278,9 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
   plan_b.init(p.ldb, lane);
   const uint32_t lds_base =
       uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)smem));  // LDS offset
-  // Along M the 32-row sub-blocks of the tile are dealt to the two wave rows alternately (wave
-  // row w owns sub-blocks w, w+2, ...), so that a short M-tile (the ragged tail of an expert)
-  // leaves both wave rows with about half of its live sub-blocks; the contraction code is
+  // Along M the 32-row sub-blocks of the tile are dealt to the wave rows in turn (wave row w
+  // owns sub-blocks w, w + WROWS, ...), so that a short M-tile (the ragged tail of an expert)
+  // leaves every wave row with about its share of the live sub-blocks; the contraction code is
   // specialised on the number of live sub-blocks of the wave.
   const int wave_row = wave / 2;
   const int wave_j = (wave % 2) * (BN / 2);
@@ -372,14 +380,14 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
         if (r < TN)
           fb[set ^ 1][r] = read_fragment<BN, B_KM>(tb, wave_j + r * 32, kk_next, tl);
         else
-          fa[set ^ 1][r - TN] = read_fragment<BM, A_KM>(ta, (2 * (r - TN) + wave_row) * 32, kk_next, tl);
+          fa[set ^ 1][r - TN] = read_fragment<BM, A_KM>(ta, (WROWS * (r - TN) + wave_row) * 32, kk_next, tl);
       };
 #pragma unroll
       for (int m = 0; m < kMfma; ++m) {
         const int i = m / TN, j = m % TN;
         acc[i][j] = Mfma<T>::run(fb[set][j], fa[set][i], acc[i][j]);
-        if ((m & 1) && reads_done < kReads) one_read(reads_done++);
-        if (m % 3 == 2 && loads_done < L1) issue_one_load(loads_done++);
+        if ((kMfma < 2 * kReads || (m & 1)) && reads_done < kReads) one_read(reads_done++);
+        if (m % (kMfma >= 3 * (L1 - L0) ? 3 : 2) == 1 && loads_done < L1) issue_one_load(loads_done++);
       }
 #pragma unroll
       for (int r = 0; r < kReads; ++r)
@@ -431,30 +439,63 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
         __builtin_amdgcn_make_buffer_rsrc(static_cast<void*>(cur.c), 0, int(uint32_t(live_rows) * row_bytes_c), 0x00020000);
     const int valid_j = cur.valid_j;
     const int r = tl % 32;
-    unsigned char* wr = buf + r * 256 + (tl / 32) * 8;
-    const int rd_row = tl / 16, rd_c16 = tl % 16;  // it-th read: row = it*4 + rd_row
+    if constexpr (kStageCols == 128) {
+      unsigned char* wr = buf + r * 256 + (tl / 32) * 8;
+      const int rd_row = tl / 16, rd_c16 = tl % 16;  // it-th read: row = it*4 + rd_row
 #pragma unroll
-    for (int i = 0; i < ATM; ++i) {
+      for (int i = 0; i < ATM; ++i) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
+        for (int j = 0; j < TN; ++j) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          Pack4<T> out;
+          for (int q = 0; q < 4; ++q) {
+            Pack4<T> out;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) out.v[e] = from_float<T>(acc[i][j][q * 4 + e]);
-          *reinterpret_cast<Pack4<T>*>(wr + (((j * 4 + q) ^ (r & 15)) * 16)) = out;
+            for (int e = 0; e < 4; ++e) out.v[e] = from_float<T>(acc[i][j][q * 4 + e]);
+            *reinterpret_cast<Pack4<T>*>(wr + (((j * 4 + q) ^ (r & 15)) * 16)) = out;
+          }
+        }
+        const int row0 = (WROWS * i + wave_row) * 32;
+        const int col = wave_j + rd_c16 * 8;
+        const bool col_live = col < valid_j;
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+          const int row = it * 4 + rd_row;
+          const uint4 v = *reinterpret_cast<const uint4*>(buf + row * 256 + ((rd_c16 ^ (row & 15)) * 16));
+          __builtin_amdgcn_raw_buffer_store_b128(
+              __builtin_bit_cast(u32x4_t, v), rsrc_c,
+              col_live ? uint32_t(row0 + row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset, 0, 0);
         }
       }
-      const int row0 = (2 * i + wave_row) * 32;
-      const int col = wave_j + rd_c16 * 8;
-      const bool col_live = col < valid_j;
+    } else {
+      // 64 columns at a time: rows of 128 bytes, 16-byte chunks swizzled with (row >> 1) & 7
+      unsigned char* wr = buf + r * 128 + (tl / 32) * 8;
+      const int rd_row = tl / 8, rd_c = tl % 8;  // it-th read: row = it*8 + rd_row
 #pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int row = it * 4 + rd_row;
-        const uint4 v = *reinterpret_cast<const uint4*>(buf + row * 256 + ((rd_c16 ^ (row & 15)) * 16));
-        __builtin_amdgcn_raw_buffer_store_b128(
-            __builtin_bit_cast(u32x4_t, v), rsrc_c,
-            col_live ? uint32_t(row0 + row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset, 0, 0);
+      for (int i = 0; i < ATM; ++i) {
+        const int row0 = (WROWS * i + wave_row) * 32;
+#pragma unroll
+        for (int round = 0; round < kColRounds; ++round) {
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              Pack4<T> out;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) out.v[e] = from_float<T>(acc[i][round * 2 + jj][q * 4 + e]);
+              *reinterpret_cast<Pack4<T>*>(wr + (((jj * 4 + q) ^ ((r >> 1) & 7)) * 16)) = out;
+            }
+          }
+          const int col = wave_j + round * 64 + rd_c * 8;
+          const bool col_live = col < valid_j;
+#pragma unroll
+          for (int it = 0; it < 4; ++it) {
+            const int row = it * 8 + rd_row;
+            const uint4 v = *reinterpret_cast<const uint4*>(buf + row * 128 + ((rd_c ^ ((row >> 1) & 7)) * 16));
+            __builtin_amdgcn_raw_buffer_store_b128(
+                __builtin_bit_cast(u32x4_t, v), rsrc_c,
+                col_live ? uint32_t(row0 + row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset, 0, 0);
+          }
+        }
       }
     }
   };
@@ -477,19 +518,29 @@ __global__ __launch_bounds__(kThreads) void persistent_gemm_kernel(GemmArgs p) {
 #pragma unroll
   for (int j = 0; j < TN; ++j) f0b[j] = read_fragment<BN, B_KM>(smem + PlanA::kStageBytes, wave_j + j * 32, 0, lane);
 #pragma unroll
-  for (int i = 0; i < TM; ++i) f0a[i] = read_fragment<BM, A_KM>(smem, (2 * i + wave_row) * 32, 0, lane);
+  for (int i = 0; i < TM; ++i) f0a[i] = read_fragment<BM, A_KM>(smem, (WROWS * i + wave_row) * 32, 0, lane);
 
   while (true) {
     const int64_t next_id = tile_id(k + wgs_per_xcd);
     const bool more = next_id >= 0;
     const int live_sub = (cur.valid_i < BM ? cur.valid_i + 31 : BM) / 32;  // live 32-row sub-blocks
-    const int my_sub = __builtin_amdgcn_readfirstlane((live_sub + 1 - wave_row) / 2);  // those of this wave row
-    switch (my_sub) {
-      case 0: run_tile(std::integral_constant<int, 0>{}, cur, more, f0a, f0b); break;
-      case 1: run_tile(std::integral_constant<int, 1>{}, cur, more, f0a, f0b); break;
-      case 2: run_tile(std::integral_constant<int, (TM >= 2 ? 2 : TM)>{}, cur, more, f0a, f0b); break;
-      case 3: run_tile(std::integral_constant<int, (TM >= 3 ? 3 : TM)>{}, cur, more, f0a, f0b); break;
-      default: run_tile(std::integral_constant<int, TM>{}, cur, more, f0a, f0b); break;
+    const int my_sub =
+        __builtin_amdgcn_readfirstlane((live_sub + WROWS - 1 - wave_row) / WROWS);  // those of this wave row
+    if constexpr (TM == 4) {
+      switch (my_sub) {
+        case 0: run_tile(std::integral_constant<int, 0>{}, cur, more, f0a, f0b); break;
+        case 1: run_tile(std::integral_constant<int, 1>{}, cur, more, f0a, f0b); break;
+        case 2: run_tile(std::integral_constant<int, 2>{}, cur, more, f0a, f0b); break;
+        case 3: run_tile(std::integral_constant<int, 3>{}, cur, more, f0a, f0b); break;
+        default: run_tile(std::integral_constant<int, 4>{}, cur, more, f0a, f0b); break;
+      }
+    } else {
+      static_assert(TM == 2, "4 or 8 waves");
+      switch (my_sub) {
+        case 0: run_tile(std::integral_constant<int, 0>{}, cur, more, f0a, f0b); break;
+        case 1: run_tile(std::integral_constant<int, 1>{}, cur, more, f0a, f0b); break;
+        default: run_tile(std::integral_constant<int, 2>{}, cur, more, f0a, f0b); break;
+      }
     }
     if (!more) break;
     k += wgs_per_xcd;
@@ -512,10 +563,10 @@ int persistent_grid() {
   return cached;
 }
 
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD>
-int launch(const GemmArgs& p, hipStream_t s) {
-  auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD>;
-  constexpr size_t smem = size_t(kStages) * (BM + BN) * kBK * 2 + size_t(kThreads / kWave) * kEpilogueScratch;
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES>
+int launch_waves(const GemmArgs& p, hipStream_t s) {
+  auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD, WAVES>;
+  constexpr size_t smem = size_t(kStages) * (BM + BN) * kBK * 2 + size_t(kEpilogueBytes);
   static bool configured = false;
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -523,8 +574,18 @@ int launch(const GemmArgs& p, hipStream_t s) {
       return STM_ERR_LAUNCH;
     configured = true;
   }
-  kernel<<<unsigned(persistent_grid()), kThreads, smem, s>>>(p);
+  kernel<<<unsigned(persistent_grid()), WAVES * kWave, smem, s>>>(p);
   return launch_status();
+}
+
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD>
+int launch(const GemmArgs& p, hipStream_t s) {
+  static const int waves = [] {
+    const char* e = getenv("STM_GEMM_WAVES");
+    return e ? atoi(e) : 8;
+  }();
+  if (waves == 4) return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, 4>(p, s);
+  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, 8>(p, s);
 }
 
 }  // namespace
