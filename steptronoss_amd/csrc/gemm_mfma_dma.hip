@@ -373,25 +373,24 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       const unsigned char* ta = smem + slot_next;
       const unsigned char* tb = ta + PlanA::kStageBytes;
       constexpr int kMfma = ATM * TN;
-      constexpr int kReads = TN + TM;  // all TM fragments are fetched: the next tile may need them
-      int reads_done = 0, loads_done = L0;
-      auto one_read = [&](int r) {
-        if (!read_next) return;
-        if (r < TN)
-          fb[set ^ 1][r] = read_fragment<BN, B_KM>(tb, wave_j + r * 32, kk_next, tl);
-        else
-          fa[set ^ 1][r - TN] = read_fragment<BM, A_KM>(ta, (WROWS * (r - TN) + wave_row) * 32, kk_next, tl);
-      };
+      int loads_done = L0;
+      // The fragments of the next slice go into the idle register set right away, in the order
+      // the next slice consumes them (A sub-block 0, then the B sub-blocks, then the other A
+      // sub-blocks), so that they have the whole slice to arrive.
+      if (read_next) {
+        fa[set ^ 1][0] = read_fragment<BM, A_KM>(ta, wave_row * 32, kk_next, tl);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[set ^ 1][j] = read_fragment<BN, B_KM>(tb, wave_j + j * 32, kk_next, tl);
+#pragma unroll
+        for (int i = 1; i < TM; ++i)
+          fa[set ^ 1][i] = read_fragment<BM, A_KM>(ta, (WROWS * i + wave_row) * 32, kk_next, tl);
+      }
 #pragma unroll
       for (int m = 0; m < kMfma; ++m) {
         const int i = m / TN, j = m % TN;
         acc[i][j] = Mfma<T>::run(fb[set][j], fa[set][i], acc[i][j]);
-        if ((kMfma < 2 * kReads || (m & 1)) && reads_done < kReads) one_read(reads_done++);
         if (m % (kMfma >= 3 * (L1 - L0) ? 3 : 2) == 1 && loads_done < L1) issue_one_load(loads_done++);
       }
-#pragma unroll
-      for (int r = 0; r < kReads; ++r)
-        if (r >= reads_done) one_read(r);
 #pragma unroll
       for (int li = L0; li < L1; ++li)
         if (li >= loads_done) issue_one_load(li);
