@@ -1,23 +1,25 @@
 // bf16 / fp16 grouped GEMM, main kernels: persistent workgroups, buffer_load ... lds (HBM/L2 ->
 // LDS without a register stop), XOR-swizzled LDS tiles, 32x32x16 MFMA.
 //
-// Shape of the design (256 x 256 output tile, contraction step 64):
-//   * one workgroup of 4 waves per CU, resident for the whole launch, walks a strided list of
-//     output tiles.  Tiles are numbered so that the workgroups of one XCD work on neighbouring
-//     tiles (same expert weights / same rows) and meet in that XCD's L2;
-//   * per step each operand tile is 256 rows x 128 B; a wave-wide load instruction moves 8 full
-//     128-byte lines (KC) or 2 x 512 contiguous bytes (KM) straight into LDS.  The CU's texture
-//     path takes about 64 cycles per such instruction, i.e. about half of a step's MFMA time
-//     for the 64 loads of a stage -- so the loads are not issued in a burst but one at a time
-//     in the shadow of the MFMAs, spread over three quarters of a step;
-//   * two LDS stages.  The (tile, step) pairs of a workgroup form ONE stream of stages: the
-//     loads of stage g+2 start as soon as every wave has read stage g, whether or not g+2
-//     belongs to the next tile, and the first MFMA fragments of a tile are fetched during the
-//     last MFMAs of the previous one; the epilogue runs while the next tile's data arrives;
+// Shape of the design (256 x 256 output tile):
+//   * one workgroup per CU (8 waves = two per SIMD, or 4), resident for the whole launch, walks
+//     a strided list of output tiles.  Tiles are numbered so that the workgroups of one XCD work
+//     on neighbouring tiles (same expert weights / same rows) and meet in that XCD's L2;
+//   * 128 KiB of LDS stages: two stages of 64 contraction elements or four of 32.  A wave-wide
+//     load instruction moves 1 KiB straight into LDS: 8 full 128-byte lines (K-contiguous
+//     operand, stages of 64), 16 half lines (stages of 32) or 2 x 512 contiguous bytes (K-major
+//     operand).  A wave pays some tens of cycles of issue time per such instruction, so the
+//     loads are not issued in a burst but one at a time in the shadow of the MFMAs, and with two
+//     waves per SIMD the other wave's MFMAs cover them;
+//   * the (tile, step) pairs of a workgroup form ONE stream of stages: the loads run ahead of
+//     the MFMAs by the number of stages, across tile boundaries, and the first MFMA fragments
+//     of a tile are fetched during the last MFMAs of the previous one; the epilogue runs while
+//     the next tile's data arrives;
 //   * raw buffer loads: anything past the end of an operand's valid region (rows past a ragged
 //     group, rows past a short M-tile) reads as zero through the bounds check, so ragged edges
 //     cost no branches;
-//   * MFMA fragments are double-buffered in registers, one LDS read per two MFMAs.
+//   * MFMA fragments are double-buffered in registers: the fragments of the next 16-wide slice
+//     are read from LDS at the start of the current one.
 //
 // The three products of the expert FFN:
 //   fwd   C = A  * W^T   A:[M,K] KC   W[g]:[N,K] KC
@@ -27,8 +29,10 @@
 // KM = operand rows are contraction steps      (read with ds_read_b64_tr_b16).
 //
 // LDS layout of one stage:
-//   KC tile: row r (128 B) at r*128, its eight 16-byte chunks stored at chunk ^ ((r >> 1) & 7):
-//            16 consecutive rows read the same logical chunk from 16 distinct bank groups.
+//   KC tile: stages of 64: row r (128 B) at r*128, its eight 16-byte chunks stored at
+//            chunk ^ ((r >> 1) & 7); stages of 32: row r (64 B) at r*64, its four chunks stored at
+//            chunk ^ ((r >> 2) & 3): 16 consecutive rows read the same logical chunk from 16
+//            distinct bank groups.
 //   KM tile: contraction row k (R*2 B) at k*R*2, its 64-byte chunks stored at chunk ^ (k & 3):
 //            the four rows a transposing read touches land in the four quarters of the banks.
 // A wave-wide buffer_load ... lds writes 1024 consecutive LDS bytes (lane l at +16*l), so the
@@ -66,8 +70,7 @@ struct Mfma<f16_t> {
   }
 };
 
-constexpr int kBK = 64;  // contraction elements per stage
-constexpr int kStages = 2;
+constexpr int kStagesBytesLog2 = 17;  // the stages of a workgroup fill 128 KiB of LDS, whatever their depth
 constexpr int kEpilogueBytes = 32768;  // output staging of all waves, behind the stages
 
 template <typename T>
@@ -101,11 +104,11 @@ __device__ __forceinline__ void dma16(i32x4_t rsrc, uint32_t lds_addr, uint32_t 
 // lane inside "its" load depends on the load index only through its parity (via the swizzle),
 // so two VGPRs per operand describe all of them; the first row of the load goes into the
 // scalar offset.
-template <int R, bool KM, int WAVES>
+template <int R, bool KM, int WAVES, int kBK>
 struct OperandPlan {
   static constexpr int kStageBytes = R * kBK * 2;  // 16-bit elements
   static constexpr int kLoadsPerWave = kStageBytes / 1024 / WAVES;
-  static constexpr int kRowsPerLoad = KM ? 1024 / (R * 2) : 8;  // stored rows covered by one load
+  static constexpr int kRowsPerLoad = KM ? 1024 / (R * 2) : 1024 / (kBK * 2);  // stored rows covered by one load
   static_assert(kLoadsPerWave % 2 == 0, "the parity trick needs an even number of loads per wave");
   static_assert(!KM || kRowsPerLoad == 2 || kRowsPerLoad == 4, "KM tiles of 128 or 256 columns");
   uint32_t voff[2];      // lane offset for even / odd loads, relative to the load's first row
@@ -117,9 +120,16 @@ struct OperandPlan {
 #pragma unroll
     for (int parity = 0; parity < 2; ++parity) {
       if constexpr (!KM) {
-        // stored row r = load*8 + lane/8, chunk = (lane%8) ^ ((r >> 1) & 7)
-        const int sw = ((parity * 4) + lane / 16) & 7;
-        voff[parity] = uint32_t(lane / 8) * row_bytes + uint32_t((lane % 8) ^ sw) * 16u;
+        if constexpr (kBK == 64) {
+          // stored row r = load*8 + lane/8 (128 bytes), chunk = (lane%8) ^ ((r >> 1) & 7)
+          const int sw = ((parity * 4) + lane / 16) & 7;
+          voff[parity] = uint32_t(lane / 8) * row_bytes + uint32_t((lane % 8) ^ sw) * 16u;
+        } else {
+          // stored row r = load*16 + lane/4 (64 bytes), chunk = (lane%4) ^ ((r >> 2) & 3): the
+          // swizzle does not depend on the load
+          const int sw = (lane / 16) & 3;
+          voff[parity] = uint32_t(lane / 4) * row_bytes + uint32_t((lane % 4) ^ sw) * 16u;
+        }
       } else {
         // stored row k = load*kRowsPerLoad + lane/(R/8), 64-byte chunk = (c16/4) ^ (k & 3)
         constexpr int kChunks16 = R / 8;
@@ -152,12 +162,12 @@ struct OperandPlan {
 };
 
 // 8 contraction values (k = kk*16 + (lane/32)*8 .. +8) of output row/column r0 + lane%32.
-template <int R, bool KM>
+template <int R, bool KM, int kBK>
 __device__ __forceinline__ uint4 read_fragment(const unsigned char* tile, int r0, int kk, int lane) {
   if constexpr (!KM) {
     const int r = r0 + lane % 32;
-    const int chunk = (kk * 2 + lane / 32) ^ ((r >> 1) & 7);
-    return *reinterpret_cast<const uint4*>(tile + r * 128 + chunk * 16);
+    const int chunk = (kk * 2 + lane / 32) ^ (kBK == 64 ? (r >> 1) & 7 : (r >> 2) & 3);
+    return *reinterpret_cast<const uint4*>(tile + r * (kBK * 2) + chunk * 16);
   } else {
     // in each 16-lane group, lanes 4r..4r+3 name stored row r (4 elements each) and lane i
     // receives column i of those four rows
@@ -183,23 +193,34 @@ struct TileState {
 // WAVES = 4: one wave per SIMD, 2 x 2 waves of 128 x 128 outputs each.
 // WAVES = 8: two waves per SIMD, 4 x 2 waves of 64 x 128 outputs each: while one wave of a SIMD
 //            sits in the issue of a load, the other one keeps the MFMA pipe busy.
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES>
+// kBK = 64: two LDS stages of 64 contraction elements (rows of 128 bytes: every load moves
+//           full lines of a K-contiguous operand);
+// kBK = 32: four stages of 32 (loads run three stages ahead: more latency hidden, but only
+//           half lines of a K-contiguous operand per row).
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int kBK>
 __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs p) {
+  static_assert(kBK == 64 || kBK == 32, "contraction elements per stage");
+  constexpr int kStages = (1 << kStagesBytesLog2) / ((BM + BN) * kBK * 2);
   constexpr int WROWS = WAVES / 2;                   // wave rows; two wave columns
   constexpr int TM = BM / 32 / WROWS, TN = BN / 64;  // 32x32 MFMA tiles per wave
   constexpr int kEpilogueScratch = kEpilogueBytes / WAVES;  // per wave: 32 rows x kStageCols outputs
   constexpr int kStageCols = kEpilogueScratch / 32 / 2;     // 128 (4 waves) or 64 (8 waves)
   constexpr int kColRounds = (BN / 2) / kStageCols;
-  using PlanA = OperandPlan<BM, A_KM, WAVES>;
-  using PlanB = OperandPlan<BN, B_KM, WAVES>;
+  using PlanA = OperandPlan<BM, A_KM, WAVES, kBK>;
+  using PlanB = OperandPlan<BN, B_KM, WAVES, kBK>;
   constexpr uint32_t kStageBytes = PlanA::kStageBytes + PlanB::kStageBytes;
   constexpr int kLoadsA = PlanA::kLoadsPerWave, kLoadsB = PlanB::kLoadsPerWave;
   constexpr int kLoads = kLoadsA + kLoadsB;  // per wave per stage
-  // where in a step the loads of later stages go out: the first kEarly loads of stage g+2 in the
-  // last quarter of step g (right after its slot is free), the rest in the first two quarters
-  // of step g+1; they have landed when step g+1 reaches its third quarter.
-  constexpr int kEarly = kLoads * 3 / 8;
+  // A step is one stage of kBK contraction elements = kBK/16 MFMA slices.  The slot of stage g
+  // is free after the barrier before the last slice of step g; the loads of stage g + kStages
+  // go out right after it: the first kEarly in the last slice of step g, the rest in the first
+  // slice(s) of step g+1 (spread over two slices when a step has four).  They are needed at the
+  // barrier of step g + kStages - 1.
+  constexpr int kEarly = kBK == 64 ? kLoads * 3 / 8 : kLoads / 2;
   constexpr int kMid = kEarly + (kLoads - kEarly + 1) / 2;
+  // loads that may still be in flight at the barrier of step g: those of stages g+2 .. g+kStages-1
+  constexpr int kInFlight = (kStages - 2) * kLoads;
+  static_assert(kInFlight < 64, "vmcnt is a 6-bit counter");
   static_assert(BN == 256 && sizeof(T) == 2 && (kStageCols == 128 || kStageCols == 64),
                 "epilogue staging assumes 128 columns of 16-bit outputs per wave, staged 128 or 64 at a time");
   extern __shared__ __align__(1024) unsigned char smem[];
@@ -296,7 +317,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   const uint32_t l_lds_b0 =
       __builtin_amdgcn_readfirstlane(lds_base + PlanA::kStageBytes + uint32_t(wave * kLoadsB) * 1024u);
   uint32_t l_soff_a = l_soff_a0, l_soff_b = l_soff_b0;
-  uint32_t l_slot = 0;  // byte offset of the LDS slot being filled: 0 or kStageBytes
+  uint32_t l_slot = 0;  // byte offset of the LDS slot being filled
   int l_step = 0, l_n_steps = 1;
   int64_t l_k = 0;
   auto load_tile = [&](const TileState<T>& t) {
@@ -322,7 +343,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     for (int li = kFirst; li < kLast; ++li) issue_one_load(li);
   };
   auto advance_loads = [&]() {  // the stage under the cursor is fully issued: move to the next
-    l_slot ^= kStageBytes;
+    l_slot = (l_slot + kStageBytes) & (kStages * kStageBytes - 1);
     l_soff_a += plan_a.step_bytes;
     l_soff_b += plan_b.step_bytes;
     if (++l_step >= l_n_steps) {
@@ -343,7 +364,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   // ---- one tile of MFMAs.  On entry the fragments of its first slice are in registers (set 0)
   // and the loads of its second stage are partly issued; on exit the same holds for the next
   // tile if there is one (`more`).
-  uint32_t c_slot = 0;  // byte offset of the LDS slot the MFMAs read: 0 or kStageBytes
+  uint32_t c_slot = 0;  // byte offset of the LDS slot the MFMAs read
   auto run_tile = [&](auto atm_tag, const TileState<T>& cur, bool more, uint4 (&f0a)[TM], uint4 (&f0b)[TN]) {
     constexpr int ATM = decltype(atm_tag)::value;
     constexpr int AR = ATM > 0 ? ATM : 1;
@@ -378,12 +399,12 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       // the next slice consumes them (A sub-block 0, then the B sub-blocks, then the other A
       // sub-blocks), so that they have the whole slice to arrive.
       if (read_next) {
-        fa[set ^ 1][0] = read_fragment<BM, A_KM>(ta, wave_row * 32, kk_next, tl);
+        fa[set ^ 1][0] = read_fragment<BM, A_KM, kBK>(ta, wave_row * 32, kk_next, tl);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fb[set ^ 1][j] = read_fragment<BN, B_KM>(tb, wave_j + j * 32, kk_next, tl);
+        for (int j = 0; j < TN; ++j) fb[set ^ 1][j] = read_fragment<BN, B_KM, kBK>(tb, wave_j + j * 32, kk_next, tl);
 #pragma unroll
         for (int i = 1; i < TM; ++i)
-          fa[set ^ 1][i] = read_fragment<BM, A_KM>(ta, (WROWS * i + wave_row) * 32, kk_next, tl);
+          fa[set ^ 1][i] = read_fragment<BM, A_KM, kBK>(ta, (WROWS * i + wave_row) * 32, kk_next, tl);
       }
 #pragma unroll
       for (int m = 0; m < kMfma; ++m) {
@@ -402,17 +423,23 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
 
     const int n_steps = cur.n_steps;
     for (int step = 0; step < n_steps; ++step) {
-      slice(0, true, c_slot, 1, CE{}, CM{});
-      slice(1, true, c_slot, 2, CM{}, CL{});
-      advance_loads();
-      slice(0, true, c_slot, 3, C0{}, C0{});
-      // everything issued so far has landed => the next stage is complete (my part); my reads
-      // of this stage are done; after the barrier that holds for the whole workgroup.  (After
-      // the last stage of the last tile this waits for empty loads and the reads below fetch
-      // fragments nobody uses: cheaper than a branch around every read.)
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      if constexpr (kBK == 64) {
+        slice(0, true, c_slot, 1, CE{}, CM{});
+        slice(1, true, c_slot, 2, CM{}, CL{});
+        advance_loads();
+        slice(0, true, c_slot, 3, C0{}, C0{});
+      } else {
+        slice(0, true, c_slot, 1, CE{}, CL{});
+        advance_loads();
+      }
+      // all but the loads of the kStages-2 youngest stages have landed => the next stage is
+      // complete (my part); my reads of this stage are done; after the barrier both hold for
+      // the whole workgroup and this stage's slot can be refilled.  (After the last stage of
+      // the last tile the loads are empty and the reads below fetch fragments nobody uses:
+      // cheaper than a branch around every read.)
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(kInFlight) : "memory");
       __syncthreads();
-      c_slot ^= kStageBytes;
+      c_slot = (c_slot + kStageBytes) & (kStages * kStageBytes - 1);
       slice(1, true, c_slot, 0, C0{}, CE{});
     }
 #pragma unroll
@@ -507,17 +534,22 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   locate(id, cur);
   l_k = k;
   load_tile(cur);
-  issue_loads(std::integral_constant<int, 0>{}, std::integral_constant<int, kLoads>{});
-  advance_loads();
+  // stages 0 .. kStages-2 in full and the head of stage kStages-1 (whose slot is free: nothing
+  // has been read yet), as the steady state has it at the start of a step
+#pragma unroll
+  for (int g = 0; g < kStages - 1; ++g) {
+    issue_loads(std::integral_constant<int, 0>{}, std::integral_constant<int, kLoads>{});
+    advance_loads();
+  }
   issue_loads(std::integral_constant<int, 0>{}, std::integral_constant<int, kEarly>{});
-  // stage 0 has landed once at most the kEarly younger loads are outstanding
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kEarly) : "memory");
+  // stage 0 has landed once at most the younger loads are outstanding
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"((kStages - 2) * kLoads + kEarly) : "memory");
   __syncthreads();
   uint4 f0a[TM], f0b[TN];
 #pragma unroll
-  for (int j = 0; j < TN; ++j) f0b[j] = read_fragment<BN, B_KM>(smem + PlanA::kStageBytes, wave_j + j * 32, 0, lane);
+  for (int j = 0; j < TN; ++j) f0b[j] = read_fragment<BN, B_KM, kBK>(smem + PlanA::kStageBytes, wave_j + j * 32, 0, lane);
 #pragma unroll
-  for (int i = 0; i < TM; ++i) f0a[i] = read_fragment<BM, A_KM>(smem, (WROWS * i + wave_row) * 32, 0, lane);
+  for (int i = 0; i < TM; ++i) f0a[i] = read_fragment<BM, A_KM, kBK>(smem, (WROWS * i + wave_row) * 32, 0, lane);
 
   while (true) {
     const int64_t next_id = tile_id(k + wgs_per_xcd);
@@ -562,10 +594,10 @@ int persistent_grid() {
   return cached;
 }
 
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES>
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int BK>
 int launch_waves(const GemmArgs& p, hipStream_t s) {
-  auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD, WAVES>;
-  constexpr size_t smem = size_t(kStages) * (BM + BN) * kBK * 2 + size_t(kEpilogueBytes);
+  auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD, WAVES, BK>;
+  constexpr size_t smem = (size_t(1) << kStagesBytesLog2) + size_t(kEpilogueBytes);
   static bool configured = false;
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -577,14 +609,14 @@ int launch_waves(const GemmArgs& p, hipStream_t s) {
   return launch_status();
 }
 
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD>
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int BK>
 int launch(const GemmArgs& p, hipStream_t s) {
   static const int waves = [] {
     const char* e = getenv("STM_GEMM_WAVES");
     return e ? atoi(e) : 8;
   }();
-  if (waves == 4) return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, 4>(p, s);
-  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, 8>(p, s);
+  if (waves == 4) return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, 4, BK>(p, s);
+  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, 8, BK>(p, s);
 }
 
 }  // namespace
@@ -595,17 +627,23 @@ constexpr int kDmaBM = 256, kDmaBN = 256;
 int launch_dma_rows(int dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap, int b_is_nk,
                     void* ws, hipStream_t s) {
   GemmArgs p = base;
-  if (p.n_k % kBK != 0 || p.n_j % 8 != 0) return STM_ERR_UNSUPPORTED;
+  if (p.n_k % 32 != 0 || p.n_j % 8 != 0) return STM_ERR_UNSUPPORTED;
   if (int64_t(p.n_k) * p.ldb * 2 >= (int64_t(1) << 32) || int64_t(kDmaBM) * p.lda * 2 >= (int64_t(1) << 32))
     return STM_ERR_UNSUPPORTED;
   const int st = build_tile_table(offsets, n_groups, kDmaBM, m_cap, ws, s);
   if (st != STM_OK) return st;
   p.tiles_j = (p.n_j + kDmaBN - 1) / kDmaBN;
-  if (dtype == STM_BF16)
-    return b_is_nk ? launch<bf16_t, kDmaBM, kDmaBN, false, false, false>(p, s)
-                   : launch<bf16_t, kDmaBM, kDmaBN, false, true, false>(p, s);
-  return b_is_nk ? launch<f16_t, kDmaBM, kDmaBN, false, false, false>(p, s)
-                 : launch<f16_t, kDmaBM, kDmaBN, false, true, false>(p, s);
+  // Both operands K-contiguous (forward): stages of 64, so that every load moves full 128-byte
+  // lines; a K-major operand in play (dgrad): four stages of 32 hide more latency.
+  const bool deep = !b_is_nk || p.n_k % 64 != 0;
+  if (dtype == STM_BF16) {
+    if (!b_is_nk) return launch<bf16_t, kDmaBM, kDmaBN, false, true, false, 32>(p, s);
+    return deep ? launch<bf16_t, kDmaBM, kDmaBN, false, false, false, 32>(p, s)
+                : launch<bf16_t, kDmaBM, kDmaBN, false, false, false, 64>(p, s);
+  }
+  if (!b_is_nk) return launch<f16_t, kDmaBM, kDmaBN, false, true, false, 32>(p, s);
+  return deep ? launch<f16_t, kDmaBM, kDmaBN, false, false, false, 32>(p, s)
+              : launch<f16_t, kDmaBM, kDmaBN, false, false, false, 64>(p, s);
 }
 
 int launch_dma_wgrad(int dtype, const GemmArgs& base, int n_groups, int64_t m_cap, hipStream_t s) {
@@ -615,8 +653,8 @@ int launch_dma_wgrad(int dtype, const GemmArgs& base, int n_groups, int64_t m_ca
   p.tiles_i = (p.n_i + kDmaBM - 1) / kDmaBM;
   p.tiles_j = (p.n_j + kDmaBN - 1) / kDmaBN;
   p.n_groups = n_groups;
-  if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, true, true, true>(p, s);
-  return launch<f16_t, kDmaBM, kDmaBN, true, true, true>(p, s);
+  if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, true, true, true, 32>(p, s);
+  return launch<f16_t, kDmaBM, kDmaBN, true, true, true, 32>(p, s);
 }
 
 }  // namespace stm
