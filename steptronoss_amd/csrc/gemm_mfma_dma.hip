@@ -37,7 +37,6 @@
 //            the four rows a transposing read touches land in the four quarters of the banks.
 // A wave-wide buffer_load ... lds writes 1024 consecutive LDS bytes (lane l at +16*l), so the
 // swizzle is applied on the global-address side.
-#include <cstdlib>
 #include <type_traits>
 
 #include "gemm_common.hpp"
@@ -231,12 +230,30 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   // below is wave-uniform and must stay on the scalar unit)
   const int64_t n_tiles = WGRAD ? int64_t(p.n_groups) * p.tiles_i * p.tiles_j
                                 : int64_t(__builtin_amdgcn_readfirstlane(p.header[0])) * p.tiles_j;
-  const int64_t per_xcd = (n_tiles + kNumXcd - 1) / kNumXcd;
+  // Normally an XCD owns a contiguous range of tile ids.  The work of a wgrad tile grows with
+  // its expert's row count; when that is very uneven (largest expert above three times the
+  // mean) a contiguous range would leave one XCD with all tiles of a large expert, so then the
+  // rows of the tile grid (tiles_j tiles sharing the A operand) are dealt to the XCDs in turn,
+  // at the price of less operand sharing in L2.
+  bool dealt = false;
+  if constexpr (WGRAD) {
+    int most = 0;
+    for (int g = threadIdx.x % kWave; g < p.n_groups; g += kWave) {
+      const int rows = p.offsets[g + 1] - p.offsets[g];
+      most = rows > most ? rows : most;
+    }
+    most = __builtin_amdgcn_readfirstlane(wave_max(most));
+    const int total = __builtin_amdgcn_readfirstlane(p.offsets[p.n_groups]);
+    dealt = int64_t(most) * p.n_groups > 3 * int64_t(total);
+  }
+  const int64_t deal = p.tiles_j;
+  const int64_t per_xcd =
+      dealt ? (n_tiles / deal + kNumXcd - 1) / kNumXcd * deal : (n_tiles + kNumXcd - 1) / kNumXcd;  // upper bound
   const int64_t xcd = blockIdx.x % kNumXcd;
   const int64_t wgs_per_xcd = gridDim.x / kNumXcd;
   auto tile_id = [&](int64_t k) -> int64_t {
     if (k >= per_xcd) return -1;
-    const int64_t id = xcd * per_xcd + k;
+    const int64_t id = dealt ? ((k / deal) * kNumXcd + xcd) * deal + k % deal : xcd * per_xcd + k;
     return id < n_tiles ? id : -1;
   };
   auto locate = [&](int64_t id, TileState<T>& t) {
@@ -609,14 +626,12 @@ int launch_waves(const GemmArgs& p, hipStream_t s) {
   return launch_status();
 }
 
+// Two waves per SIMD: measured faster than one (4 waves) on every product of the expert FFN.
+constexpr int kGemmWaves = 8;
+
 template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int BK>
 int launch(const GemmArgs& p, hipStream_t s) {
-  static const int waves = [] {
-    const char* e = getenv("STM_GEMM_WAVES");
-    return e ? atoi(e) : 8;
-  }();
-  if (waves == 4) return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, 4, BK>(p, s);
-  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, 8, BK>(p, s);
+  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, kGemmWaves, BK>(p, s);
 }
 
 }  // namespace
