@@ -1,0 +1,154 @@
+"""The hot path at the full sizes of the benchmark configurations (c2, c3, c4), checked through
+properties that do not need an oracle run of that size: permutations are permutations, stable
+and expert-sorted; permuted rows are bit-exact copies; permute -> combine with unit weights
+multiplies by K exactly; sampled rows / experts / tokens of the GEMMs and of the whole layer
+agree with fp32 torch arithmetic on the same rounded inputs (rel-L2 <= 1e-2 for bf16)."""
+
+import pytest
+import torch
+
+import bench
+from tests.helpers import rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+TOL = 1e-2  # bf16 storage, fp32 accumulation
+
+
+@pytest.fixture(scope="module", params=["c2", "c3", "c4"])
+def case(request):
+    from steptronoss_amd.model.common.moe_block import forward_router
+
+    cfg = bench.WORKLOADS[request.param]
+    torch.cuda.set_device(DEV)
+    x, w1, w2, logits, go = bench.make_inputs(cfg, 1234, DEV)
+    ids, weights, aux, hist = forward_router(
+        logits, cfg["K"], use_sigmoid=cfg["sigmoid"], norm_expert_weight=cfg["norm"], n_group=cfg["n_group"],
+        topk_group=cfg["topk_group"],
+    )  # fmt: skip
+    yield dict(name=request.param, cfg=cfg, x=x, w1=w1, w2=w2, logits=logits, go=go, ids=ids, weights=weights, aux=aux, hist=hist)
+    del x, w1, w2, logits, go
+    torch.cuda.empty_cache()
+
+
+def test_router_invariants(case):
+    cfg, ids, weights, hist = case["cfg"], case["ids"], case["weights"], case["hist"]
+    T, E, K = cfg["T"], cfg["E"], cfg["K"]
+    assert ids.shape == (T, K) and ids.dtype == torch.int64
+    assert int(ids.min()) >= 0 and int(ids.max()) < E
+    srt = ids.sort(dim=1).values
+    assert bool((srt[:, 1:] != srt[:, :-1]).all()), "an expert was picked twice for a token"
+    assert torch.equal(hist.long(), torch.bincount(ids.reshape(-1), minlength=E))
+    assert int(hist.sum()) == T * K
+    assert float((weights.sum(1) - 1).abs().max()) < 1e-5  # renormalised
+    assert bool((weights[:, 1:] <= weights[:, :-1] + 1e-7).all()), "weights are not in selection order"
+    if cfg["n_group"] > 1:
+        groups = ids // (E // cfg["n_group"])
+        n_groups_used = torch.zeros(T, cfg["n_group"], device=DEV).scatter_(1, groups, 1.0).sum(1)
+        assert int(n_groups_used.max()) <= cfg["topk_group"]
+    if case["name"] == "c3":  # the skewed configuration must really be skewed
+        assert int(hist.max()) > 5 * T * K // E
+    aux_ref = (torch.softmax(case["logits"].float(), 1) if not cfg["sigmoid"] else None)
+    if aux_ref is not None:
+        expect = float((aux_ref.mean(0) * hist.float()).sum() * E)
+        assert abs(float(case["aux"]) - expect) <= 1e-4 * abs(expect)
+
+
+def test_route_plan_is_the_stable_expert_sort(case):
+    from steptronoss_amd.model.utils import moe_utils as M
+
+    cfg, ids = case["cfg"], case["ids"]
+    E, N = cfg["E"], ids.numel()
+    hist, offsets, pos, _ = M.route_plan(ids, E)
+    assert torch.equal(hist, case["hist"].to(hist.dtype))
+    assert torch.equal(offsets[1:].long(), torch.cumsum(hist.long(), 0)) and int(offsets[0]) == 0
+    flat = pos.reshape(-1).long()
+    inv = torch.full((N,), -1, device=DEV, dtype=torch.long)
+    inv[flat] = torch.arange(N, device=DEV)
+    assert int(inv.min()) >= 0, "positions are not a permutation of 0..N-1"
+    e_sorted = ids.reshape(-1)[inv]
+    nondecreasing = e_sorted[1:] >= e_sorted[:-1]
+    stable = (e_sorted[1:] > e_sorted[:-1]) | (inv[1:] > inv[:-1])
+    assert bool(nondecreasing.all()) and bool(stable.all())
+    # the stand-alone ops give the same answer
+    assert torch.equal(M.index_compute(ids, M.histogram(ids, E)), pos)
+
+
+def test_permute_is_an_exact_copy_and_round_trips(case):
+    from steptronoss_amd.model.utils import moe_utils as M
+
+    cfg, x, ids = case["cfg"], case["x"], case["ids"]
+    K = cfg["K"]
+    pos = M.index_compute(ids, case["hist"])
+    xg = x.detach().clone().requires_grad_(True)
+    xp = M.moe_scatter(xg, pos)
+    assert xp.shape == (ids.numel(), x.shape[1])
+    for k in range(K):  # row pos[t,k] holds token t, bit for bit
+        assert torch.equal(xp.detach()[pos[:, k].long()], x)
+    ones = torch.ones(ids.shape, device=DEV, dtype=torch.float32)
+    back = M.moe_weighted_gather(xp, pos, ones)
+    assert torch.equal(back.detach().float(), x.float() * K)  # K is a power of two: exact in bf16
+    back.backward(torch.ones_like(back))
+    assert torch.equal(xg.grad.float(), torch.full_like(x, float(K * 1)).float())
+
+
+def test_grouped_gemm_samples_match_fp32(case):
+    from steptronoss_amd.model.utils import moe_utils as M
+
+    cfg, x, w1, ids = case["cfg"], case["x"], case["w1"], case["ids"]
+    E = cfg["E"]
+    hist, offsets, pos, _ = M.route_plan(ids, E)
+    xp = M.moe_scatter(x, pos).detach().requires_grad_(True)
+    w = w1.detach().requires_grad_(True)
+    out = M.grouped_gemm(xp, w, hist.long(), trans_b=True)
+    gen = torch.Generator(device=DEV).manual_seed(7)
+    go = torch.randn(out.shape, device=DEV, generator=gen).to(out.dtype)
+    out.backward(go)
+    off = offsets.long().cpu()
+    sizes = (off[1:] - off[:-1])
+    busiest = int(sizes.argmax())
+    smallest_live = int(torch.where(sizes > 0, sizes, sizes.max() + 1).argmin())
+    for e in {0, E // 2, E - 1, busiest, smallest_live}:
+        lo, hi = int(off[e]), int(off[e + 1])
+        if hi == lo:
+            assert float(w.grad[e].abs().sum()) == 0.0  # an expert without rows gets a zero gradient
+            continue
+        rows = torch.arange(lo, hi, device=DEV)[torch.linspace(0, hi - lo - 1, min(64, hi - lo)).long().to(DEV)]
+        ref = xp.detach()[rows].float() @ w1[e].float().t()
+        assert rel_l2(out.detach()[rows], ref) <= TOL
+        ref_da = go[rows].float() @ w1[e].float()
+        assert rel_l2(xp.grad[rows], ref_da) <= TOL
+        ref_dw = go[lo:hi].float().t() @ xp.detach()[lo:hi].float()
+        assert rel_l2(w.grad[e], ref_dw) <= TOL
+    empty = torch.nonzero(sizes == 0).reshape(-1)
+    if empty.numel():
+        assert float(w.grad[empty.to(DEV)].abs().sum()) == 0.0
+
+
+def test_layer_samples_match_fp32(case):
+    from steptronoss_amd.model.common.feed_forward import swiglu
+    from steptronoss_amd.model.utils import moe_utils as M
+
+    cfg, x, w1, w2, ids, weights, go = (case[k] for k in ("cfg", "x", "w1", "w2", "ids", "weights", "go"))
+    xg = x.detach().requires_grad_(True)
+    a, b = w1.detach().requires_grad_(True), w2.detach().requires_grad_(True)
+    tw = weights.detach().requires_grad_(True)
+    out = M.routed_grouped_ffn(a, b, swiglu, xg, ids, tw)
+    out.backward(go)
+    F = cfg["F"]
+    for t in torch.linspace(0, cfg["T"] - 1, 6).long().tolist():
+        xt = x[t].float().clone().requires_grad_(True)
+        wt = weights[t].detach().clone().requires_grad_(True)
+        acc = torch.zeros(x.shape[1], device=DEV)
+        for k in range(cfg["K"]):
+            e = int(ids[t, k])
+            gu = (w1[e].float() @ xt).to(x.dtype).float()  # the layer stores gate/up in bf16
+            h = (torch.nn.functional.silu(gu[:F]) * gu[F:]).to(x.dtype).float()
+            y = (w2[e].float() @ h).to(x.dtype).float()
+            acc = acc + wt[k] * y
+        acc.backward(go[t].float())
+        assert rel_l2(out.detach()[t], acc.detach()) <= TOL
+        assert rel_l2(tw.grad[t], wt.grad) <= 2 * TOL
+        assert rel_l2(xg.grad[t], xt.grad) <= 2 * TOL
+    assert a.grad.shape == w1.shape and b.grad.shape == w2.shape
+    assert bool(torch.isfinite(a.grad).all()) and bool(torch.isfinite(b.grad).all())
