@@ -20,6 +20,23 @@ __device__ __forceinline__ int64_t load_pos(const void* pos, int64_t i) {
     return static_cast<const int32_t*>(pos)[i];
 }
 
+// The gather kernels take the slots of a token in batches of kBatch: first all positions, then
+// all row loads (unconditional, from row 0 for a slot that is not routed, so that the loads of
+// a batch are in flight together), then the arithmetic in slot order.
+constexpr int kBatch = 8;
+
+template <bool I64>
+__device__ __forceinline__ void load_batch(const void* pos, int64_t slot0, int k0, int top_k, int64_t n_rows,
+                                           int64_t (&row)[kBatch], bool (&ok)[kBatch]) {
+#pragma unroll
+  for (int c = 0; c < kBatch; ++c) {
+    const int k = k0 + c;
+    const int64_t p = k < top_k ? load_pos<I64>(pos, slot0 + k) : -1;
+    ok[c] = p >= 0 && p < n_rows;
+    row[c] = ok[c] ? p : 0;
+  }
+}
+
 // ---------------------------------------------------------------- permute forward
 // Bit copy; V is the widest unit that divides the row and the base alignment.
 template <typename V, bool I64>
@@ -97,16 +114,24 @@ __global__ __launch_bounds__(kRowThreads) void permute_bwd_kernel(const T* __res
   const int64_t t = blockIdx.x;
   const int64_t units = hidden / VEC;
   const int64_t slot0 = t * top_k;
+  if (n_rows == 0) top_k = 0;  // nothing to gather from
   for (int64_t u = threadIdx.x; u < units; u += kRowThreads) {
     float acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-    for (int k = 0; k < top_k; ++k) {
-      const int64_t p = load_pos<I64>(pos, slot0 + k);
-      if (p < 0 || p >= n_rows) continue;
-      const P row = reinterpret_cast<const P*>(go + p * hidden)[u];
+    for (int k0 = 0; k0 < top_k; k0 += kBatch) {
+      int64_t row[kBatch];
+      bool ok[kBatch];
+      load_batch<I64>(pos, slot0, k0, top_k, n_rows, row, ok);
+      P v[kBatch];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] += to_float(row.v[j]);
+      for (int c = 0; c < kBatch; ++c) v[c] = reinterpret_cast<const P*>(go + row[c] * hidden)[u];
+#pragma unroll
+      for (int c = 0; c < kBatch; ++c) {
+        if (!ok[c]) continue;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += to_float(v[c].v[j]);
+      }
     }
     P o;
 #pragma unroll
@@ -128,20 +153,28 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_fwd_kernel(const T* __r
   const int64_t t = blockIdx.x;
   const int64_t units = hidden / VEC;
   const int64_t slot0 = t * top_k;
+  if (n_rows == 0) top_k = 0;  // nothing to gather from
   for (int64_t u = threadIdx.x; u < units; u += kRowThreads) {
     float acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-    for (int k = 0; k < top_k; ++k) {
-      const int64_t p = load_pos<I64>(pos, slot0 + k);
-      if (p < 0 || p >= n_rows) continue;
-      float w = load_weight_any(weight, wdtype, slot0 + k);
-      if constexpr (!FP32W) w = round_through<T>(w);
-      const P row = reinterpret_cast<const P*>(in + p * hidden)[u];
+    for (int k0 = 0; k0 < top_k; k0 += kBatch) {
+      int64_t row[kBatch];
+      bool ok[kBatch];
+      load_batch<I64>(pos, slot0, k0, top_k, n_rows, row, ok);
+      P v[kBatch];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float prod = to_float(row.v[j]) * w;
-        acc[j] += FP32W ? prod : round_through<T>(prod);
+      for (int c = 0; c < kBatch; ++c) v[c] = reinterpret_cast<const P*>(in + row[c] * hidden)[u];
+#pragma unroll
+      for (int c = 0; c < kBatch; ++c) {
+        if (!ok[c]) continue;
+        float w = load_weight_any(weight, wdtype, slot0 + k0 + c);
+        if constexpr (!FP32W) w = round_through<T>(w);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float prod = to_float(v[c].v[j]) * w;
+          acc[j] += FP32W ? prod : round_through<T>(prod);
+        }
       }
     }
     P o;
@@ -154,7 +187,7 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_fwd_kernel(const T* __r
 // ---------------------------------------------------------------- unpermute backward
 // grad_in[pos[t,k],:] = go[t,:] * w[t,k] (both rounded to T), grad_w[t,k] = <go[t,:], in[pos,:]>
 // (fp32 accumulation).  Valid for an injective pos: each row is written by one slot.
-constexpr int kDotChunk = 8;
+constexpr int kDotChunk = kBatch;
 
 template <typename T, int VEC, bool I64>
 __global__ __launch_bounds__(kRowThreads) void unpermute_bwd_kernel(
@@ -164,7 +197,7 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_bwd_kernel(
   using P = Pack<T, VEC>;
   __shared__ float partial[kRowThreads / kWave][kDotChunk];
   const int64_t t = blockIdx.x;
-  const int64_t units = hidden / VEC;
+  const int64_t units = n_rows > 0 ? hidden / VEC : 0;  // no rows: nothing to read, d weight = 0
   const int64_t slot0 = t * top_k;
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
@@ -174,22 +207,24 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_bwd_kernel(
     for (int c = 0; c < kDotChunk; ++c) dot[c] = 0.f;
     for (int64_t u = threadIdx.x; u < units; u += kRowThreads) {
       const P g = reinterpret_cast<const P*>(go + t * hidden)[u];
+      int64_t row[kBatch];
+      bool ok[kBatch];
+      load_batch<I64>(pos, slot0, k0, top_k, n_rows, row, ok);
+      P v[kBatch];
 #pragma unroll
-      for (int c = 0; c < kDotChunk; ++c) {
-        const int k = k0 + c;
-        if (k >= top_k) break;
-        const int64_t p = load_pos<I64>(pos, slot0 + k);
-        if (p < 0 || p >= n_rows) continue;
-        const float w = round_through<T>(load_weight_any(weight, wdtype, slot0 + k));
-        const P row = reinterpret_cast<const P*>(in + p * hidden)[u];
+      for (int c = 0; c < kBatch; ++c) v[c] = reinterpret_cast<const P*>(in + row[c] * hidden)[u];
+#pragma unroll
+      for (int c = 0; c < kBatch; ++c) {
+        if (!ok[c]) continue;
+        const float w = round_through<T>(load_weight_any(weight, wdtype, slot0 + k0 + c));
         P o;
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
           const float gj = to_float(g.v[j]);
-          dot[c] += gj * to_float(row.v[j]);
+          dot[c] += gj * to_float(v[c].v[j]);
           o.v[j] = from_float<T>(gj * w);
         }
-        reinterpret_cast<P*>(gin + p * hidden)[u] = o;
+        reinterpret_cast<P*>(gin + row[c] * hidden)[u] = o;
       }
     }
 #pragma unroll
