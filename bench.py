@@ -174,10 +174,9 @@ def main():
 
     timing = kt.summary()
     e = 2  # bytes per bf16 element
-    gemm = timing.get("stm_grouped_gemm", {"calls": 0, "total_ms": 0.0})
-    wgrad = timing.get("stm_grouped_gemm_wgrad", {"calls": 0, "total_ms": 0.0})
-    gemm_calls = gemm["calls"] + wgrad["calls"]
-    gemm_ms = gemm["total_ms"] + wgrad["total_ms"]
+    gemm_entries = ("stm_grouped_gemm", "stm_grouped_gemm_wgrad", "stm_grouped_gemm_swiglu", "stm_grouped_gemm_dswiglu")
+    gemm_calls = sum(timing[n]["calls"] for n in gemm_entries if n in timing)
+    gemm_ms = sum(timing[n]["total_ms"] for n in gemm_entries if n in timing)
     # six equal-cost-per-flop launches per step: 4 over [N, H] x 2F-sized problems count double
     flops_per_launch = flops / 6.0
     avg_launch_ms = gemm_ms / max(gemm_calls, 1)
@@ -213,6 +212,7 @@ def main():
         "swiglu_fwd_us": timing.get("stm_swiglu_fwd", {}).get("avg_us"),
         "swiglu_bwd_us": timing.get("stm_swiglu_bwd", {}).get("avg_us"),
     }
+    entry_us = {name: round(t["avg_us"], 1) for name, t in sorted(timing.items())}
 
     result = {
         "metric": METRIC,
@@ -241,6 +241,7 @@ def main():
         "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS,
         "roofline": roofline,
         "bandwidth": bandwidth,
+        "entry_avg_us": entry_us,
     }
     if not args.no_cpu_baseline:
         threads = min(os.cpu_count() or 1, 16)

@@ -185,6 +185,23 @@ size_t stm_gemm_workspace_bytes(int64_t m_cap, int n_groups);
 int stm_grouped_gemm(const void* a, const void* b, void* c, const int32_t* offsets, int n_groups, int64_t m_cap, int n,
                      int k, int b_is_nk, int dtype, void* workspace, size_t workspace_bytes, stm_stream_t stream);
 
+/* The two products of the expert FFN that touch the SwiGLU, with the SwiGLU done in the GEMM's
+ * epilogue (routed_grouped_ffn, moe_utils.py:237-241, with act = feed_forward.py:20-26):
+ *   stm_grouped_gemm_swiglu : gate_up [m_cap, 2*ffn] = a [m_cap, k] * w1[g]^T (w1 [G, 2*ffn, k])
+ *                             and h [m_cap, ffn] = swiglu(gate_up), both stored;
+ *   stm_grouped_gemm_dswiglu: d gate_up [m_cap, 2*ffn] from d h = grad_y [m_cap, k] * w2[g]
+ *                             (w2 [G, k, ffn]) and gate_up; d h itself is never stored.
+ * Results are bit-identical to stm_grouped_gemm followed by stm_swiglu_fwd / stm_swiglu_bwd.
+ * Return STM_ERR_UNSUPPORTED for shapes the fused kernels do not take (k not a multiple of 32,
+ * ffn not a multiple of 8, fewer than 4096 rows, fp32): callers then use the unfused pair.
+ * Workspace as for stm_grouped_gemm. */
+int stm_grouped_gemm_swiglu(const void* a, const void* w1, void* gate_up, void* h, const int32_t* offsets, int n_groups,
+                            int64_t m_cap, int ffn, int k, int has_limit, float limit, int dtype, void* workspace,
+                            size_t workspace_bytes, stm_stream_t stream);
+int stm_grouped_gemm_dswiglu(const void* grad_y, const void* w2, const void* gate_up, void* grad_gate_up,
+                             const int32_t* offsets, int n_groups, int64_t m_cap, int ffn, int k, int has_limit,
+                             float limit, int dtype, void* workspace, size_t workspace_bytes, stm_stream_t stream);
+
 /* grouped_gemm wgrad, function_imple.py:54-69: out[g] = x[rows of g]^T @ y[rows of g],
  * x:[m_cap, p], y:[m_cap, q], out:[G, p, q]; an empty group gives zeros (:56-58). */
 int stm_grouped_gemm_wgrad(const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,

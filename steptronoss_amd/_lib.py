@@ -56,6 +56,8 @@ SIGNATURES = {
     "stm_gemm_workspace_bytes": (Z, [L, I]),
     "stm_grouped_gemm": (I, [P, P, P, P, I, L, I, I, I, I, P, Z, P]),
     "stm_grouped_gemm_wgrad": (I, [P, P, P, P, I, L, I, I, I, P]),
+    "stm_grouped_gemm_swiglu": (I, [P, P, P, P, P, I, L, I, I, I, F, I, P, Z, P]),
+    "stm_grouped_gemm_dswiglu": (I, [P, P, P, P, P, I, L, I, I, I, F, I, P, Z, P]),
     "stm_swiglu_fwd": (I, [P, P, L, L, P, I, F, I, P]),
     "stm_swiglu_bwd": (I, [P, P, P, L, L, P, I, F, I, P]),
     "stm_router_workspace_bytes": (Z, [L, I]),
@@ -119,6 +121,24 @@ def call(name: str, *args) -> None:
         hook.after(name, token)
     if code != 0:
         raise RuntimeError(f"{name} failed: {status_string(code)} (status {code})")
+
+
+ERR_UNSUPPORTED = -2
+
+
+def try_call(name: str, *args) -> bool:
+    """Like :func:`call` for entry points that may decline a shape: ``False`` when the library
+    answers "unsupported" (the caller then takes another entry point), raises on real errors."""
+    hook = _call_hook
+    token = hook.before(name) if hook is not None else None
+    code = getattr(load(), name)(*args)
+    if hook is not None:
+        hook.after(name, token)
+    if code == ERR_UNSUPPORTED:
+        return False
+    if code != 0:
+        raise RuntimeError(f"{name} failed: {status_string(code)} (status {code})")
+    return True
 
 
 def ptr(t: torch.Tensor | None):

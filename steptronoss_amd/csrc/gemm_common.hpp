@@ -51,7 +51,21 @@ struct GemmArgs {
   int tiles_i, tiles_j;
   int n_groups;
   int64_t blocks_padded;
+  // SwiGLU fused into the epilogue (rows form only):
+  //   forward:  c = gate_up [M, 2*ffn] and c2 = h [M, ffn] are both written;
+  //   backward: the product is d h; c2 = gate_up is read, c = d gate_up [M, 2*ffn] is written.
+  void* c2;
+  int64_t ldc2;
+  int ffn;
+  int has_limit;
+  float limit;
 };
+
+// Fused SwiGLU forms of the rows GEMM (gemm_mfma_dma.hip); STM_ERR_UNSUPPORTED when the shape does not fit.
+int launch_dma_swiglu_fwd(int dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap,
+                          void* ws, hipStream_t s);
+int launch_dma_swiglu_bwd(int dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap,
+                          void* ws, hipStream_t s);
 
 // Enqueue the kernel that fills the table for tiles of height bm (defined in gemm_generic.hip).
 int build_tile_table(const int32_t* offsets, int n_groups, int bm, int64_t m_cap, void* table, hipStream_t stream);

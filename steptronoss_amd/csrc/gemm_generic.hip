@@ -199,6 +199,70 @@ int stm_grouped_gemm(const void* a, const void* b, void* c, const int32_t* offse
   return dispatch_generic(dtype, p, grid, s);
 }
 
+namespace {
+// Common checks and argument block of the two fused entries.
+int fused_args(const void* a, const void* b, void* c, void* c2, const int32_t* offsets, int n_groups, int64_t m_cap,
+               int ffn, int k, int has_limit, float limit, int dtype, void* workspace, size_t workspace_bytes,
+               stm::GemmArgs& p) {
+  using namespace stm;
+  if (n_groups < 0 || m_cap < 0 || ffn < 0 || k < 0) return STM_ERR_ARG;
+  if ((dtype != STM_BF16 && dtype != STM_F16) || n_groups > kMaxGroups) return STM_ERR_UNSUPPORTED;
+  if (m_cap < 4096 || ffn == 0 || k == 0 || n_groups == 0) return STM_ERR_UNSUPPORTED;  // the unfused path handles it
+  if (!a || !b || !c || !c2 || !offsets || !workspace) return STM_ERR_ARG;
+  if (workspace_bytes < stm_gemm_workspace_bytes(m_cap, n_groups)) return STM_ERR_WORKSPACE;
+  if (!aligned_to(a, 16) || !aligned_to(b, 16) || !aligned_to(c, 16) || !aligned_to(c2, 16)) return STM_ERR_UNSUPPORTED;
+  p = GemmArgs{};
+  p.a = a;
+  p.b = b;
+  p.c = c;
+  p.c2 = c2;
+  p.offsets = offsets;
+  p.header = static_cast<const int32_t*>(workspace);
+  p.tiles = reinterpret_cast<const MTile*>(static_cast<const char*>(workspace) + 16);
+  p.n_groups = n_groups;
+  p.ffn = ffn;
+  p.has_limit = has_limit;
+  p.limit = limit;
+  return STM_OK;
+}
+}  // namespace
+
+int stm_grouped_gemm_swiglu(const void* a, const void* w1, void* gate_up, void* h, const int32_t* offsets, int n_groups,
+                            int64_t m_cap, int ffn, int k, int has_limit, float limit, int dtype, void* workspace,
+                            size_t workspace_bytes, stm_stream_t stream) {
+  using namespace stm;
+  GemmArgs p;
+  const int st = fused_args(a, w1, gate_up, h, offsets, n_groups, m_cap, ffn, k, has_limit, limit, dtype, workspace,
+                            workspace_bytes, p);
+  if (st != STM_OK) return st;
+  p.lda = k;
+  p.ldb = k;
+  p.ldc = 2 * int64_t(ffn);
+  p.ldc2 = ffn;
+  p.b_group = 2 * int64_t(ffn) * k;
+  p.n_j = 2 * ffn;
+  p.n_k = k;
+  return launch_dma_swiglu_fwd(dtype, p, offsets, n_groups, m_cap, workspace, as_stream(stream));
+}
+
+int stm_grouped_gemm_dswiglu(const void* grad_y, const void* w2, const void* gate_up, void* grad_gate_up,
+                             const int32_t* offsets, int n_groups, int64_t m_cap, int ffn, int k, int has_limit,
+                             float limit, int dtype, void* workspace, size_t workspace_bytes, stm_stream_t stream) {
+  using namespace stm;
+  GemmArgs p;
+  const int st = fused_args(grad_y, w2, grad_gate_up, const_cast<void*>(gate_up), offsets, n_groups, m_cap, ffn, k,
+                            has_limit, limit, dtype, workspace, workspace_bytes, p);
+  if (st != STM_OK) return st;
+  p.lda = k;
+  p.ldb = ffn;  // w2[g] is [k, ffn]: contraction rows, K-major for this product
+  p.ldc = 2 * int64_t(ffn);
+  p.ldc2 = 2 * int64_t(ffn);
+  p.b_group = int64_t(ffn) * k;
+  p.n_j = ffn;
+  p.n_k = k;
+  return launch_dma_swiglu_bwd(dtype, p, offsets, n_groups, m_cap, workspace, as_stream(stream));
+}
+
 int stm_grouped_gemm_wgrad(const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
                            int64_t m_cap, int p_dim, int q_dim, int dtype, stm_stream_t stream) {
   using namespace stm;

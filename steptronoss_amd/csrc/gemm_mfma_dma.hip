@@ -40,6 +40,7 @@
 #include <type_traits>
 
 #include "gemm_common.hpp"
+#include "swiglu_math.hpp"
 
 namespace stm {
 namespace {
@@ -76,6 +77,14 @@ template <typename T>
 struct alignas(sizeof(T) * 4) Pack4 {
   T v[4];
 };
+template <typename T>
+struct alignas(sizeof(T) * 8) Pack8 {
+  T v[8];
+};
+template <typename T>
+__device__ __forceinline__ float round_to(float f) {
+  return to_float(from_float<T>(f));
+}
 
 // Raw buffer descriptor over [base, base + bytes): reads past the end return zero.
 __device__ __forceinline__ i32x4_t make_rsrc(const void* base, uint32_t bytes) {
@@ -186,8 +195,14 @@ template <typename T>
 struct TileState {
   i32x4_t rsrc_a, rsrc_b;
   T* c;
+  T* c2;             // second output / extra input of a fused epilogue (first row of the tile)
+  uint32_t soff_b0;  // scalar offset of this wave's first B load of a stage at contraction step 0
+  int col0;          // first output column of the tile (fused SwiGLU: first gate column)
   int valid_i, valid_j, n_steps;
 };
+
+// What the epilogue does with the accumulators.
+enum Epilogue { kStore = 0, kSwigluFwd = 1, kSwigluBwd = 2 };
 
 // WAVES = 4: one wave per SIMD, 2 x 2 waves of 128 x 128 outputs each.
 // WAVES = 8: two waves per SIMD, 4 x 2 waves of 64 x 128 outputs each: while one wave of a SIMD
@@ -196,9 +211,18 @@ struct TileState {
 //           full lines of a K-contiguous operand);
 // kBK = 32: four stages of 32 (loads run three stages ahead: more latency hidden, but only
 //           half lines of a K-contiguous operand per row).
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int kBK>
+// EPI = kSwigluFwd (C = A * W1^T, both K-contiguous): a tile holds 128 gate columns and the 128
+//   up columns that go with them, interleaved in blocks of 64 (gate c..c+63 | up c..c+63 | gate
+//   c+64.. | up c+64..), so that a lane finds gate and up of one output element in its own
+//   accumulators; gate_up is stored in its usual [gate | up] layout and h = swiglu(gate_up)
+//   beside it, both rounded as the unfused kernels round them.
+// EPI = kSwigluBwd (d h = d y * W2): d h is never stored; the epilogue reads gate_up and stores
+//   d gate_up.
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int kBK, int EPI>
 __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs p) {
   static_assert(kBK == 64 || kBK == 32, "contraction elements per stage");
+  static_assert(EPI == kStore || (WAVES == 8 && !WGRAD && !A_KM), "fused epilogues: rows form, 8 waves");
+  static_assert(EPI != kSwigluFwd || !B_KM, "the fused forward reads W1 rows K-contiguous");
   constexpr int kStages = (1 << kStagesBytesLog2) / ((BM + BN) * kBK * 2);
   constexpr int WROWS = WAVES / 2;                   // wave rows; two wave columns
   constexpr int TM = BM / 32 / WROWS, TN = BN / 64;  // 32x32 MFMA tiles per wave
@@ -256,15 +280,22 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     const int64_t id = dealt ? ((k / deal) * kNumXcd + xcd) * deal + k % deal : xcd * per_xcd + k;
     return id < n_tiles ? id : -1;
   };
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int lane = threadIdx.x % kWave;
+  // rows of B a wave loads per stage start at tile row wave * (BN / WAVES)
+  const uint32_t b_rows_per_wave = BN / WAVES;
   auto locate = [&](int64_t id, TileState<T>& t) {
     const T* a = static_cast<const T*>(p.a);
     const T* b = static_cast<const T*>(p.b);
     T* c = static_cast<T*>(p.c);
     const int jt = int(id % p.tiles_j);
-    const int j0 = jt * BN;
+    const int j0 = EPI == kSwigluFwd ? jt * (BN / 2) : jt * BN;
     int n_k;
     uint32_t a_bytes, b_bytes;
-    t.valid_j = p.n_j - j0;
+    t.valid_j = (EPI == kSwigluFwd ? p.ffn : p.n_j) - j0;
+    t.col0 = j0;
+    t.c2 = nullptr;
+    t.soff_b0 = 0;
     if constexpr (WGRAD) {
       const int64_t rest = id / p.tiles_j;
       const int it = int(rest % p.tiles_i);
@@ -290,9 +321,19 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       n_k = p.n_k;
       t.valid_i = mt.rows;
       a += int64_t(mt.row0) * p.lda;
-      c += int64_t(mt.row0) * p.ldc + j0;
+      c += int64_t(mt.row0) * p.ldc + (EPI == kStore ? j0 : 0);
+      if constexpr (EPI != kStore) t.c2 = static_cast<T*>(p.c2) + int64_t(mt.row0) * p.ldc2;
       a_bytes = uint32_t(int64_t(mt.rows) * p.lda * 2);
-      if constexpr (B_KM) {
+      if constexpr (EPI == kSwigluFwd) {
+        // the descriptor covers all 2*ffn rows of the expert's W1; this wave's 32 tile rows are
+        // one run of gate rows or of up rows
+        const uint32_t seg = uint32_t(wave) * b_rows_per_wave / 64u;  // 0: gate, 1: up, 2: gate + 64, 3: up + 64
+        const uint32_t w_row = (seg & 1u ? uint32_t(p.ffn) : 0u) + uint32_t(j0) + (seg >> 1) * 64u +
+                               uint32_t(wave) * b_rows_per_wave % 64u;
+        b += int64_t(mt.group) * p.b_group;
+        b_bytes = uint32_t(int64_t(2 * p.ffn) * p.ldb * 2);
+        t.soff_b0 = __builtin_amdgcn_readfirstlane(w_row * uint32_t(p.ldb * 2));
+      } else if constexpr (B_KM) {
         b += int64_t(mt.group) * p.b_group + j0;
         b_bytes = uint32_t(int64_t(p.n_k) * p.ldb * 2 - int64_t(j0) * 2);
       } else {
@@ -308,8 +349,6 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     t.n_steps = __builtin_amdgcn_readfirstlane(steps > 0 ? steps : 1);
   };
 
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int lane = threadIdx.x % kWave;
   PlanA plan_a;
   PlanB plan_b;
   plan_a.init(p.lda, lane);
@@ -329,7 +368,8 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   // keeps going with an empty descriptor: such loads move no data (and write zeros to an LDS
   // slot nobody reads any more), which keeps the steady-state code free of branches.
   i32x4_t l_rsrc_a, l_rsrc_b;
-  const uint32_t l_soff_a0 = plan_a.stage_soffset(0, wave), l_soff_b0 = plan_b.stage_soffset(0, wave);
+  const uint32_t l_soff_a0 = plan_a.stage_soffset(0, wave);
+  uint32_t l_soff_b0 = plan_b.stage_soffset(0, wave);  // per tile for the fused forward
   const uint32_t l_lds_a0 = __builtin_amdgcn_readfirstlane(lds_base + uint32_t(wave * kLoadsA) * 1024u);
   const uint32_t l_lds_b0 =
       __builtin_amdgcn_readfirstlane(lds_base + PlanA::kStageBytes + uint32_t(wave * kLoadsB) * 1024u);
@@ -345,6 +385,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     }
     l_n_steps = __builtin_amdgcn_readfirstlane(t.n_steps);
     l_step = 0;
+    if constexpr (EPI == kSwigluFwd) l_soff_b0 = __builtin_amdgcn_readfirstlane(t.soff_b0);
     l_soff_a = l_soff_a0;
     l_soff_b = l_soff_b0;
   };
@@ -513,30 +554,111 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       // 64 columns at a time: rows of 128 bytes, 16-byte chunks swizzled with (row >> 1) & 7
       unsigned char* wr = buf + r * 128 + (tl / 32) * 8;
       const int rd_row = tl / 8, rd_c = tl % 8;  // it-th read: row = it*8 + rd_row
+      // one round: 32 rows x 64 values, rounded to T, from the accumulators into the scratch ...
+      auto stage = [&](auto&& value) {  // value(jj, q, e): column jj*32 + q*8 + (lane/32)*4 + e of this lane's row
 #pragma unroll
-      for (int i = 0; i < ATM; ++i) {
-        const int row0 = (WROWS * i + wave_row) * 32;
+        for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
-        for (int round = 0; round < kColRounds; ++round) {
+          for (int q = 0; q < 4; ++q) {
+            Pack4<T> out;
 #pragma unroll
-          for (int jj = 0; jj < 2; ++jj) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              Pack4<T> out;
-#pragma unroll
-              for (int e = 0; e < 4; ++e) out.v[e] = from_float<T>(acc[i][round * 2 + jj][q * 4 + e]);
-              *reinterpret_cast<Pack4<T>*>(wr + (((jj * 4 + q) ^ ((r >> 1) & 7)) * 16)) = out;
-            }
+            for (int e = 0; e < 4; ++e) out.v[e] = from_float<T>(value(jj, q, e));
+            *reinterpret_cast<Pack4<T>*>(wr + (((jj * 4 + q) ^ ((r >> 1) & 7)) * 16)) = out;
           }
-          const int col = wave_j + round * 64 + rd_c * 8;
-          const bool col_live = col < valid_j;
+        }
+      };
+      // ... and back: 8 consecutive values of row it*8 + rd_row, columns rd_c*8 .. +7
+      auto staged = [&](int it) {
+        const int row = it * 8 + rd_row;
+        return *reinterpret_cast<const uint4*>(buf + row * 128 + ((rd_c ^ ((row >> 1) & 7)) * 16));
+      };
+      if constexpr (EPI == kStore) {
 #pragma unroll
-          for (int it = 0; it < 4; ++it) {
-            const int row = it * 8 + rd_row;
-            const uint4 v = *reinterpret_cast<const uint4*>(buf + row * 128 + ((rd_c ^ ((row >> 1) & 7)) * 16));
-            __builtin_amdgcn_raw_buffer_store_b128(
-                __builtin_bit_cast(u32x4_t, v), rsrc_c,
-                col_live ? uint32_t(row0 + row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset, 0, 0);
+        for (int i = 0; i < ATM; ++i) {
+          const int row0 = (WROWS * i + wave_row) * 32;
+#pragma unroll
+          for (int round = 0; round < kColRounds; ++round) {
+            stage([&](int jj, int q, int e) { return acc[i][round * 2 + jj][q * 4 + e]; });
+            const int col = wave_j + round * 64 + rd_c * 8;
+            const bool col_live = col < valid_j;
+#pragma unroll
+            for (int it = 0; it < 4; ++it)
+              __builtin_amdgcn_raw_buffer_store_b128(
+                  __builtin_bit_cast(u32x4_t, staged(it)), rsrc_c,
+                  col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset, 0,
+                  0);
+          }
+        }
+      } else {
+        const bool has_limit = p.has_limit != 0;
+        const float limit = p.limit;
+        const uint32_t row_bytes_2 = uint32_t(p.ldc2) * 2u;
+        const __amdgpu_buffer_rsrc_t rsrc_2 = __builtin_amdgcn_make_buffer_rsrc(
+            static_cast<void*>(cur.c2), 0, int(uint32_t(live_rows) * row_bytes_2), 0x00020000);
+        const uint32_t up_bytes = uint32_t(p.ffn) * 2u;  // from a gate column to its up column
+        if constexpr (EPI == kSwigluFwd) {
+          // accumulator tiles 0,1 of this wave: 64 gate columns; tiles 2,3: their up columns
+          const int col = cur.col0 + (wave % 2) * 64 + rd_c * 8;  // gate column = column of h
+          const bool col_live = rd_c * 8 + (wave % 2) * 64 < valid_j;
+#pragma unroll
+          for (int i = 0; i < ATM; ++i) {
+            const int row0 = (WROWS * i + wave_row) * 32;
+            auto store_round = [&](__amdgpu_buffer_rsrc_t rsrc, uint32_t row_bytes, uint32_t byte0) {
+#pragma unroll
+              for (int it = 0; it < 4; ++it)
+                __builtin_amdgcn_raw_buffer_store_b128(
+                    __builtin_bit_cast(u32x4_t, staged(it)), rsrc,
+                    col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes + byte0 + uint32_t(col) * 2u : kDroppedOffset,
+                    0, 0);
+            };
+            stage([&](int jj, int q, int e) { return acc[i][jj][q * 4 + e]; });
+            store_round(rsrc_c, row_bytes_c, 0u);
+            stage([&](int jj, int q, int e) { return acc[i][2 + jj][q * 4 + e]; });
+            store_round(rsrc_c, row_bytes_c, up_bytes);
+            stage([&](int jj, int q, int e) {  // from the values as stored: h = swiglu(rounded gate, rounded up)
+              return swiglu_value(round_to<T>(acc[i][jj][q * 4 + e]), round_to<T>(acc[i][2 + jj][q * 4 + e]), has_limit,
+                                  limit);
+            });
+            store_round(rsrc_2, row_bytes_2, 0u);
+          }
+        } else {
+          // the accumulators hold d h; gate and up come from gate_up (c2), d gate | d up go to c
+#pragma unroll
+          for (int i = 0; i < ATM; ++i) {
+            const int row0 = (WROWS * i + wave_row) * 32;
+#pragma unroll
+            for (int round = 0; round < kColRounds; ++round) {
+              const int col = cur.col0 + wave_j + round * 64 + rd_c * 8;
+              const bool col_live = wave_j + round * 64 + rd_c * 8 < valid_j;
+              uint4 gate[4], up[4];
+#pragma unroll
+              for (int it = 0; it < 4; ++it) {
+                const uint32_t at =
+                    col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes_2 + uint32_t(col) * 2u : kDroppedOffset;
+                gate[it] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_2, at, 0, 0));
+                up[it] = __builtin_bit_cast(
+                    uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_2, col_live ? at + up_bytes : kDroppedOffset, 0, 0));
+              }
+              stage([&](int jj, int q, int e) { return acc[i][round * 2 + jj][q * 4 + e]; });
+#pragma unroll
+              for (int it = 0; it < 4; ++it) {
+                const uint4 d = staged(it);
+                Pack8<T> dv = __builtin_bit_cast(Pack8<T>, d), gv = __builtin_bit_cast(Pack8<T>, gate[it]),
+                         uv = __builtin_bit_cast(Pack8<T>, up[it]), og, ou;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                  float dg, du;
+                  swiglu_grads(to_float(gv.v[e]), to_float(uv.v[e]), to_float(dv.v[e]), has_limit, limit, dg, du);
+                  og.v[e] = from_float<T>(dg);
+                  ou.v[e] = from_float<T>(du);
+                }
+                const uint32_t at =
+                    col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset;
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, og), rsrc_c, at, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, ou), rsrc_c,
+                                                       col_live ? at + up_bytes : kDroppedOffset, 0, 0);
+              }
+            }
           }
         }
       }
@@ -611,9 +733,9 @@ int persistent_grid() {
   return cached;
 }
 
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int BK>
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int BK, int EPI>
 int launch_waves(const GemmArgs& p, hipStream_t s) {
-  auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD, WAVES, BK>;
+  auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD, WAVES, BK, EPI>;
   constexpr size_t smem = (size_t(1) << kStagesBytesLog2) + size_t(kEpilogueBytes);
   static bool configured = false;
   if (!configured) {
@@ -629,9 +751,9 @@ int launch_waves(const GemmArgs& p, hipStream_t s) {
 // Two waves per SIMD: measured faster than one (4 waves) on every product of the expert FFN.
 constexpr int kGemmWaves = 8;
 
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int BK>
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int BK, int EPI = kStore>
 int launch(const GemmArgs& p, hipStream_t s) {
-  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, kGemmWaves, BK>(p, s);
+  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, kGemmWaves, BK, EPI>(p, s);
 }
 
 }  // namespace
@@ -659,6 +781,41 @@ int launch_dma_rows(int dtype, const GemmArgs& base, const int32_t* offsets, int
   if (!b_is_nk) return launch<f16_t, kDmaBM, kDmaBN, false, true, false, 32>(p, s);
   return deep ? launch<f16_t, kDmaBM, kDmaBN, false, false, false, 32>(p, s)
               : launch<f16_t, kDmaBM, kDmaBN, false, false, false, 64>(p, s);
+}
+
+// gate_up = a * w1^T with h = swiglu(gate_up) written by the same kernel.  base: a, b = w1
+// [G, 2*ffn, k], c = gate_up, c2 = h, n_k, ffn, limit filled in.
+int launch_dma_swiglu_fwd(int dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap,
+                          void* ws, hipStream_t s) {
+  GemmArgs p = base;
+  if (p.n_k % 32 != 0 || p.ffn % 8 != 0 || p.ffn < 64) return STM_ERR_UNSUPPORTED;
+  if (int64_t(2 * p.ffn) * p.ldb * 2 >= (int64_t(1) << 32) || int64_t(kDmaBM) * p.lda * 2 >= (int64_t(1) << 32))
+    return STM_ERR_UNSUPPORTED;
+  const int st = build_tile_table(offsets, n_groups, kDmaBM, m_cap, ws, s);
+  if (st != STM_OK) return st;
+  p.tiles_j = (p.ffn + kDmaBN / 2 - 1) / (kDmaBN / 2);
+  const bool deep = p.n_k % 64 != 0;
+  if (dtype == STM_BF16)
+    return deep ? launch<bf16_t, kDmaBM, kDmaBN, false, false, false, 32, kSwigluFwd>(p, s)
+                : launch<bf16_t, kDmaBM, kDmaBN, false, false, false, 64, kSwigluFwd>(p, s);
+  return deep ? launch<f16_t, kDmaBM, kDmaBN, false, false, false, 32, kSwigluFwd>(p, s)
+              : launch<f16_t, kDmaBM, kDmaBN, false, false, false, 64, kSwigluFwd>(p, s);
+}
+
+// d gate_up from d y * w2 (= d h, never stored) and gate_up.  base: a = d y, b = w2 [G, k, ffn],
+// c = d gate_up, c2 = gate_up, n_k, ffn, limit filled in.
+int launch_dma_swiglu_bwd(int dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap,
+                          void* ws, hipStream_t s) {
+  GemmArgs p = base;
+  if (p.n_k % 32 != 0 || p.ffn % 8 != 0) return STM_ERR_UNSUPPORTED;
+  if (int64_t(p.n_k) * p.ldb * 2 >= (int64_t(1) << 32) || int64_t(kDmaBM) * p.lda * 2 >= (int64_t(1) << 32))
+    return STM_ERR_UNSUPPORTED;
+  const int st = build_tile_table(offsets, n_groups, kDmaBM, m_cap, ws, s);
+  if (st != STM_OK) return st;
+  p.n_j = p.ffn;
+  p.tiles_j = (p.ffn + kDmaBN - 1) / kDmaBN;
+  if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, false, true, false, 32, kSwigluBwd>(p, s);
+  return launch<f16_t, kDmaBM, kDmaBN, false, true, false, 32, kSwigluBwd>(p, s);
 }
 
 int launch_dma_wgrad(int dtype, const GemmArgs& base, int n_groups, int64_t m_cap, hipStream_t s) {

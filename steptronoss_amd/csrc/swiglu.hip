@@ -1,7 +1,7 @@
 // SwiGLU between the two expert GEMMs: h = silu(gate) * up with gate = gu[:, :F], up = gu[:, F:],
 // optional clamp (gate side from above after the SiLU, up side to [-limit, limit]); and its
 // backward.  Element-wise, 128-bit accesses, fp32 math, one rounding per output.
-#include "common.hpp"
+#include "swiglu_math.hpp"
 
 namespace stm {
 namespace {
@@ -10,8 +10,6 @@ template <typename T, int VEC>
 struct alignas(sizeof(T) * VEC) Pack {
   T v[VEC];
 };
-
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + __expf(-x)); }
 
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const T* __restrict__ gu, T* __restrict__ h, int64_t rows,
@@ -28,14 +26,7 @@ __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const T* __restrict__ g
     P o;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      const float gv = to_float(g.v[j]);
-      float a = gv * sigmoidf_(gv);
-      float b = to_float(u.v[j]);
-      if (has_limit) {
-        a = fminf(a, limit);
-        b = fminf(fmaxf(b, -limit), limit);
-      }
-      o.v[j] = from_float<T>(a * b);
+      o.v[j] = from_float<T>(swiglu_value(to_float(g.v[j]), to_float(u.v[j]), has_limit, limit));
     }
     *reinterpret_cast<P*>(h + r * f + c) = o;
   }
@@ -58,21 +49,10 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ g
     P og, ou;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      const float gv = to_float(g.v[j]);
-      const float s = sigmoidf_(gv);
-      float a = gv * s;
-      float da = s * (1.f + gv * (1.f - s));
-      float b = to_float(u.v[j]);
-      float db = 1.f;
-      if (has_limit) {
-        if (a > limit) da = 0.f;  // clamp passes the gradient on [.., limit]
-        a = fminf(a, limit);
-        if (b < -limit || b > limit) db = 0.f;
-        b = fminf(fmaxf(b, -limit), limit);
-      }
-      const float dv = to_float(d.v[j]);
-      og.v[j] = from_float<T>(dv * b * da);
-      ou.v[j] = from_float<T>(dv * a * db);
+      float dg, du;
+      swiglu_grads(to_float(g.v[j]), to_float(u.v[j]), to_float(d.v[j]), has_limit, limit, dg, du);
+      og.v[j] = from_float<T>(dg);
+      ou.v[j] = from_float<T>(du);
     }
     *reinterpret_cast<P*>(dgu + r * 2 * f + c) = og;
     *reinterpret_cast<P*>(dgu + r * 2 * f + f + c) = ou;

@@ -25,7 +25,7 @@ from dataclasses import dataclass
 import torch
 
 from steptronoss_amd import _lib
-from steptronoss_amd._lib import call, dtype_code, is_i64, ptr, require_gpu, stream
+from steptronoss_amd._lib import call, try_call, dtype_code, is_i64, ptr, require_gpu, stream
 from steptronoss_amd.utils.optimizable import optimizable
 
 BACKEND_NAME = "hip_gfx950"
@@ -503,6 +503,36 @@ class _CombineInjective(torch.autograd.Function):
         return grad_rows, None, gw
 
 
+def _gemm_swiglu_rows(a: torch.Tensor, w1: torch.Tensor, offsets: torch.Tensor, swiglu_limit):
+    """``gate_up = a @ w1[g]^T`` and ``h = swiglu(gate_up)`` from one kernel; ``(None, None)``
+    when the fused kernel does not take the shape."""
+    m_cap, k = a.shape
+    n_groups, two_f, _ = w1.shape
+    ffn = two_f // 2
+    gu = torch.empty((m_cap, two_f), device=a.device, dtype=a.dtype)
+    h = torch.empty((m_cap, ffn), device=a.device, dtype=a.dtype)
+    ws = _gemm_workspace(m_cap, n_groups, a.device)
+    ok = try_call(
+        "stm_grouped_gemm_swiglu", ptr(a), ptr(w1), ptr(gu), ptr(h), ptr(offsets), n_groups, m_cap, ffn, k,
+        int(swiglu_limit is not None), float(swiglu_limit or 0.0), dtype_code(a.dtype), ptr(ws), ws.numel(), stream(),
+    )  # fmt: skip
+    return (gu, h) if ok else (None, None)
+
+
+def _gemm_dswiglu_rows(gy: torch.Tensor, w2: torch.Tensor, gu: torch.Tensor, offsets: torch.Tensor, swiglu_limit):
+    """``d gate_up`` from ``d h = gy @ w2[g]`` and ``gate_up`` in one kernel (``d h`` is never
+    stored); ``None`` when the fused kernel does not take the shape."""
+    m_cap, k = gy.shape
+    n_groups, _, ffn = w2.shape
+    dgu = torch.empty_like(gu)
+    ws = _gemm_workspace(m_cap, n_groups, gy.device)
+    ok = try_call(
+        "stm_grouped_gemm_dswiglu", ptr(gy), ptr(w2), ptr(gu), ptr(dgu), ptr(offsets), n_groups, m_cap, ffn, k,
+        int(swiglu_limit is not None), float(swiglu_limit or 0.0), dtype_code(gy.dtype), ptr(ws), ws.numel(), stream(),
+    )  # fmt: skip
+    return dgu if ok else None
+
+
 class _FusedRoutedFFN(torch.autograd.Function):
     """route_plan -> permute -> GEMM(w1^T) -> SwiGLU -> GEMM(w2^T) -> combine in one autograd
     node: no host round trip, intermediates are sized for all ``T*K`` slots and only the rows of
@@ -526,8 +556,10 @@ class _FusedRoutedFFN(torch.autograd.Function):
             call(
                 "stm_permute_fwd", ptr(x), ptr(pos), 0, ptr(xp), T, K, H * x.element_size(), n_rows, None, stream()
             )
-            gu = _gemm_rows(xp, w1, offsets, two_f, True)
-            h = swiglu_fwd_rows(gu, swiglu_limit, live)
+            gu, h = _gemm_swiglu_rows(xp, w1, offsets, swiglu_limit)
+            if h is None:
+                gu = _gemm_rows(xp, w1, offsets, two_f, True)
+                h = swiglu_fwd_rows(gu, swiglu_limit, live)
             y = _gemm_rows(h, w2, offsets, H, True)
             out = _combine_rows(y, pos, token_weights)
         ctx.save_for_backward(w1, w2, xp, gu, h, y, pos, offsets, token_weights)
@@ -552,8 +584,10 @@ class _FusedRoutedFFN(torch.autograd.Function):
             if need_w2:
                 gw2 = _gemm_wgrad(gy, h, offsets, E)
             if need_w1 or need_x:
-                dh = _gemm_rows(gy, w2, offsets, h.shape[1], False)
-                dgu = swiglu_bwd_rows(gu, dh, ctx.limit, live)
+                dgu = _gemm_dswiglu_rows(gy, w2, gu, offsets, ctx.limit)
+                if dgu is None:
+                    dh = _gemm_rows(gy, w2, offsets, h.shape[1], False)
+                    dgu = swiglu_bwd_rows(gu, dh, ctx.limit, live)
                 if need_w1:
                     gw1 = _gemm_wgrad(dgu, xp, offsets, E)
                 if need_x:

@@ -98,3 +98,47 @@ def test_argument_errors():
         M.grouped_gemm(a, torch.zeros(2, 8, 12, device=DEV), torch.tensor([2, 2]), trans_b=True)
     with pytest.raises(TypeError):
         M.grouped_gemm(a, torch.zeros(2, 8, 16, device=DEV, dtype=torch.bfloat16), torch.tensor([2, 2]), trans_b=True)
+
+
+# ----- SwiGLU fused into the GEMM epilogues: same bits as the GEMM followed by the SwiGLU kernel
+@pytest.mark.parametrize("limit", [None, 0.75])
+@pytest.mark.parametrize(
+    "sizes,k,ffn,dtype",
+    [
+        ([1000, 0, 37, 2500, 300, 900], 256, 192, torch.bfloat16),  # ragged groups, an empty one, half-used column tile
+        ([513, 2047, 1536], 96, 768, torch.bfloat16),  # contraction a multiple of 32 only
+        ([4096, 256], 128, 72, torch.float16),  # narrow FFN: most of a tile's columns unused
+    ],
+)
+def test_fused_swiglu_epilogues_match_the_unfused_pair(sizes, k, ffn, dtype, limit):
+    from steptronoss_amd.model.common.feed_forward import swiglu_bwd_rows, swiglu_fwd_rows
+
+    gen = torch.Generator().manual_seed(9)
+    E, m = len(sizes), sum(sizes)
+    a = torch.randn(m, k, generator=gen).to(dtype).to(DEV)
+    w1 = (torch.randn(E, 2 * ffn, k, generator=gen) * 0.2).to(dtype).to(DEV)
+    w2 = (torch.randn(E, k, ffn, generator=gen) * 0.2).to(dtype).to(DEV)
+    gy = torch.randn(m, k, generator=gen).to(dtype).to(DEV)
+    offsets = M._group_offsets(torch.tensor(sizes), torch.device(DEV))
+    gu, h = M._gemm_swiglu_rows(a, w1, offsets, limit)
+    assert h is not None, "the fused kernel declined a shape it should take"
+    gu_ref = M._gemm_rows(a, w1, offsets, 2 * ffn, True)
+    h_ref = swiglu_fwd_rows(gu_ref, limit)
+    assert torch.equal(gu, gu_ref)
+    assert torch.equal(h, h_ref)
+    dgu = M._gemm_dswiglu_rows(gy, w2, gu_ref, offsets, limit)
+    assert dgu is not None
+    dh_ref = M._gemm_rows(gy, w2, offsets, ffn, False)
+    dgu_ref = swiglu_bwd_rows(gu_ref, dh_ref, limit)
+    assert torch.equal(dgu, dgu_ref)
+    # and against the oracle in fp32
+    ref32 = O.swiglu(O.grouped_gemm(a.cpu().float(), w1.cpu().float(), torch.tensor(sizes), trans_b=True), limit)
+    assert rel_l2(h, ref32) <= 1e-2
+
+
+def test_fused_swiglu_declines_small_or_odd_shapes():
+    dev = torch.device(DEV)
+    a = torch.randn(64, 40, device=dev).bfloat16()
+    w1 = torch.randn(2, 48, 40, device=dev).bfloat16()
+    offsets = M._group_offsets(torch.tensor([30, 34]), dev)
+    assert M._gemm_swiglu_rows(a, w1, offsets, None) == (None, None)  # fewer than 4096 rows, k % 32 != 0
