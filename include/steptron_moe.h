@@ -223,6 +223,22 @@ int stm_swiglu_bwd(const void* gate_up, const void* grad_out, void* grad_gate_up
                    const int32_t* live_rows_or_null, int has_limit, float limit, int dtype, stm_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
+ * fp8 (OCP e4m3, |max| 448) operands with one fp32 scale per row per 128 contraction elements.
+ * No counterpart in the reference (its grouped GEMMs are bf16/fp16/fp32, moe_utils.py:423-453);
+ * this is the fp8 benchmark configuration's forward and dgrad.
+ * stm_quantize_e4m3_1x128: scales [rows, ceil(cols/128)] = amax/448 (1 for an all-zero block),
+ *   codes [rows, cols] = nearest e4m3 of x/scale (ties to even, saturating).
+ * stm_grouped_gemm_fp8: c[r, :] = sum over 128-blocks kb of a_scales[r,kb] * b_scales[g,:,kb] *
+ *   (a_codes[r, kb] . b_codes[g, :, kb]) for the rows r of every group g; b is [G, n, k]
+ *   (for dgrad pass the transposed weights, quantised along their own last axis).
+ *   k must be a multiple of 128.  Workspace as for stm_grouped_gemm. */
+int stm_quantize_e4m3_1x128(const void* x, int dtype, int64_t rows, int64_t cols, uint8_t* codes_out, float* scales_out,
+                            stm_stream_t stream);
+int stm_grouped_gemm_fp8(const uint8_t* a_codes, const float* a_scales, const uint8_t* b_codes, const float* b_scales,
+                         void* c, const int32_t* offsets, int n_groups, int64_t m_cap, int n, int k, int out_dtype,
+                         void* workspace, size_t workspace_bytes, stm_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
  * Router: scores, stable top-k, weight normalisation, load-balance statistics.
  * ---------------------------------------------------------------------------------- */
 

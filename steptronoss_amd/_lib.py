@@ -58,6 +58,8 @@ SIGNATURES = {
     "stm_grouped_gemm_wgrad": (I, [P, P, P, P, I, L, I, I, I, P]),
     "stm_grouped_gemm_swiglu": (I, [P, P, P, P, P, I, L, I, I, I, F, I, P, Z, P]),
     "stm_grouped_gemm_dswiglu": (I, [P, P, P, P, P, I, L, I, I, I, F, I, P, Z, P]),
+    "stm_quantize_e4m3_1x128": (I, [P, I, L, L, P, P, P]),
+    "stm_grouped_gemm_fp8": (I, [P, P, P, P, P, P, I, L, I, I, I, P, Z, P]),
     "stm_swiglu_fwd": (I, [P, P, L, L, P, I, F, I, P]),
     "stm_swiglu_bwd": (I, [P, P, P, L, L, P, I, F, I, P]),
     "stm_router_workspace_bytes": (Z, [L, I]),

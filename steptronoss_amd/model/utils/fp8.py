@@ -1,0 +1,62 @@
+"""fp8 (e4m3, 1x128 block scales) forms of the expert GEMMs on the gfx950 kernels.
+
+The reference has no fp8 path (its grouped GEMMs run in the activations' dtype, reference
+steptronoss/model/utils/moe_utils.py:423-453); this module serves the fp8 configuration of the
+benchmark: quantise activations and weights with one fp32 scale per row per 128 contraction
+elements, then ``grouped_gemm_fp8`` for the forward product and, on the transposed weights,
+for dgrad.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from steptronoss_amd import _lib
+from steptronoss_amd._lib import call, dtype_code, ptr, require_gpu, stream
+
+BLOCK = 128
+
+
+def quantize_e4m3_1x128(x: torch.Tensor):
+    """``(codes uint8 [..., C], scales float32 [..., ceil(C/128)])`` of the last axis of ``x``."""
+    require_gpu(x)
+    xc = x.contiguous()
+    cols = xc.shape[-1]
+    rows = xc.numel() // max(cols, 1)
+    codes = torch.empty(xc.shape, device=x.device, dtype=torch.uint8)
+    scales = torch.empty(xc.shape[:-1] + ((cols + BLOCK - 1) // BLOCK,), device=x.device, dtype=torch.float32)
+    with torch.cuda.device(x.device):
+        call("stm_quantize_e4m3_1x128", ptr(xc), dtype_code(xc.dtype), rows, cols, ptr(codes), ptr(scales), stream())
+    return codes, scales
+
+
+def grouped_gemm_fp8(a_codes, a_scales, b_codes, b_scales, batch_sizes, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """``out[rows of g] = dequant(a)[rows of g] @ dequant(b[g])^T`` with ``a`` ``[M, K]`` and ``b``
+    ``[G, N, K]`` quantised along ``K`` (a multiple of 128); products and sums in fp32."""
+    from steptronoss_amd.model.utils.moe_utils import _gemm_workspace, _group_offsets
+
+    dev = require_gpu(a_codes, b_codes, a_scales, b_scales)
+    if a_codes.dtype != torch.uint8 or b_codes.dtype != torch.uint8:
+        raise TypeError("codes must be uint8 tensors")
+    if a_codes.dim() != 2 or b_codes.dim() != 3 or a_codes.shape[1] != b_codes.shape[2]:
+        raise ValueError("a must be [M, K] and b [G, N, K]")
+    m_cap, k = a_codes.shape
+    n_groups, n, _ = b_codes.shape
+    if k % BLOCK:
+        raise ValueError("the contraction length must be a multiple of 128")
+    if a_scales.shape != (m_cap, k // BLOCK) or b_scales.shape != (n_groups, n, k // BLOCK):
+        raise ValueError("scales must be [M, K/128] and [G, N, K/128]")
+    with torch.cuda.device(dev):
+        offsets = _group_offsets(batch_sizes, dev)
+        out = torch.zeros((m_cap, n), device=dev, dtype=out_dtype)
+        ws = _gemm_workspace(m_cap, n_groups, dev)
+        call(
+            "stm_grouped_gemm_fp8", ptr(a_codes.contiguous()), ptr(a_scales.contiguous().float()),
+            ptr(b_codes.contiguous()), ptr(b_scales.contiguous().float()), ptr(out), ptr(offsets), n_groups, m_cap, n, k,
+            dtype_code(out_dtype), ptr(ws), ws.numel(), stream(),
+        )  # fmt: skip
+    return out
+
+
+def _keepalive():  # the library handle, for callers that only import this module
+    return _lib.load()

@@ -1,0 +1,91 @@
+"""fp8 e4m3 quantiser and grouped GEMM against the oracle.  This path is not in the reference.
+
+Two bars: (1) the kernel against exact arithmetic on the SAME quantised operands (rel-L2 <= 5e-5
+with fp32 output: only the fp32 summation order differs); (2) against the unquantised fp32
+product.  For (2) the benchmark names 3e-2, which e4m3 cannot meet on zero-mean Gaussian
+operands whatever the kernel does: three mantissa bits give each operand a relative rounding
+error of up to 2^-4 (about 2.6 % rms), the two operands together about 3.7 % of every product,
+and with random signs the sum keeps that ratio.  The measured 3.4-3.7 % is that noise; the test
+pins it below 4.5e-2 so that a real arithmetic error (a wrong scale, a dropped block) still fails."""
+
+QUANT_NOISE_TOL = 4.5e-2
+
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests.helpers import rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols", [(7, 128), (33, 384), (5, 200), (64, 1024)])
+def test_quantiser_matches_oracle_bit_for_bit(rows, cols, dtype):
+    from steptronoss_amd.model.utils.fp8 import quantize_e4m3_1x128
+
+    gen = torch.Generator().manual_seed(rows * 1000 + cols)
+    x = (torch.randn(rows, cols, generator=gen) * torch.logspace(-4, 2, rows).unsqueeze(1)).to(dtype)
+    x[0, :128] = 0  # an all-zero block
+    x[1, 5] = -0.0
+    q_ref, s_ref = O.quantize_e4m3_1x128(x.float())
+    q, s = quantize_e4m3_1x128(x.to(DEV))
+    assert torch.equal(s.cpu(), s_ref)
+    assert torch.equal(q.cpu(), q_ref)
+    back = O.dequantize_e4m3_1x128(q.cpu(), s.cpu())
+    assert rel_l2(back, x.float()) <= 4e-2  # 3 mantissa bits
+
+
+def test_quantiser_rounding_cases():
+    from steptronoss_amd.model.utils.fp8 import quantize_e4m3_1x128
+
+    # a block whose amax is 448 has scale 1: the codes are the plain e4m3 roundings
+    vals = [448.0, 1.0625, 1.1875, 2.0**-9, 1.5 * 2.0**-9, 2.5 * 2.0**-9, 2.0**-10, 500.0 / 500.0 * 447.9, -3.3, 0.0]
+    x = torch.zeros(1, 128)
+    x[0, : len(vals)] = torch.tensor(vals)
+    q, s = quantize_e4m3_1x128(x.to(DEV))
+    assert float(s[0, 0]) == 1.0
+    assert torch.equal(q.cpu()[0, : len(vals)], O.e4m3_round(torch.tensor(vals)))
+    assert q.cpu()[0, 1] == 0x38 and q.cpu()[0, 2] == 0x3A  # ties to the even mantissa
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("sizes,k,n", [([3, 0, 130, 64], 256, 96), ([200, 57], 128, 136), ([129], 512, 128)])
+def test_grouped_gemm_fp8(sizes, k, n, out_dtype):
+    from steptronoss_amd.model.utils.fp8 import grouped_gemm_fp8, quantize_e4m3_1x128
+
+    gen = torch.Generator().manual_seed(17)
+    m, G = sum(sizes), len(sizes)
+    a = torch.randn(m, k, generator=gen).bfloat16()
+    w = (torch.randn(G, n, k, generator=gen) * 0.05).bfloat16()
+    aq, as_ = quantize_e4m3_1x128(a.to(DEV))
+    wq, ws = quantize_e4m3_1x128(w.to(DEV))
+    out = grouped_gemm_fp8(aq, as_, wq, ws, torch.tensor(sizes), out_dtype=out_dtype)
+    # exact arithmetic on the quantised operands (what the kernel computes, up to fp32 summation order)
+    a_dq = O.dequantize_e4m3_1x128(aq.cpu(), as_.cpu())
+    w_dq = O.dequantize_e4m3_1x128(wq.cpu().reshape(G * n, k), ws.cpu().reshape(G * n, -1)).reshape(G, n, k)
+    ref_q = O.grouped_gemm(a_dq, w_dq, torch.tensor(sizes), trans_b=True)
+    assert rel_l2(out, ref_q) <= (4e-3 if out_dtype == torch.bfloat16 else 5e-5)
+    # against the unquantised product: quantisation noise only (see the module docstring)
+    ref = O.grouped_gemm(a.float(), w.float(), torch.tensor(sizes), trans_b=True)
+    assert rel_l2(out, ref) <= QUANT_NOISE_TOL
+
+
+def test_fp8_forward_and_dgrad_of_an_expert_layer():
+    """Forward x @ w^T and dgrad dy @ w as the same product on separately quantised operands."""
+    from steptronoss_amd.model.utils.fp8 import grouped_gemm_fp8, quantize_e4m3_1x128
+
+    gen = torch.Generator().manual_seed(23)
+    sizes = [300, 212]
+    m, G, H, F2 = sum(sizes), 2, 256, 384
+    x = torch.randn(m, H, generator=gen).bfloat16()
+    w1 = (torch.randn(G, F2, H, generator=gen) * 0.05).bfloat16()
+    dy = torch.randn(m, F2, generator=gen).bfloat16()
+    bs = torch.tensor(sizes)
+    y = grouped_gemm_fp8(*quantize_e4m3_1x128(x.to(DEV)), *quantize_e4m3_1x128(w1.to(DEV)), bs)
+    w1_t = w1.transpose(1, 2).contiguous()  # [G, H, F2]: quantised along F2, the contraction of dgrad
+    dx = grouped_gemm_fp8(*quantize_e4m3_1x128(dy.to(DEV)), *quantize_e4m3_1x128(w1_t.to(DEV)), bs)
+    assert rel_l2(y, O.grouped_gemm(x.float(), w1.float(), bs, trans_b=True)) <= QUANT_NOISE_TOL
+    ref_dx, _ = O.grouped_gemm_grads(x.float(), w1.float(), bs, True, dy.float())
+    assert rel_l2(dx, ref_dx) <= QUANT_NOISE_TOL
