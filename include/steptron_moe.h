@@ -267,6 +267,12 @@ int stm_router_bwd(const void* logits, int logits_dtype, int64_t n_tokens, int n
                    int norm_weights, float eps, const int64_t* ids, const float* grad_weights,
                    const float* grad_aux_or_null, const int32_t* hist, void* grad_logits, stm_stream_t stream);
 
+/* Aux-loss-free load balancing, one MoE layer: bias[e] += sign(mean(tokens) - tokens[e]) * rate
+ * (fp32 bias; sign(0) = 0), then tokens[e] = 0 if zero_tokens
+ * (MoEBlock.update_router_balance_bias_per_gbs, moe_block.py:442-491, after its all-reduces). */
+int stm_router_bias_update(int32_t* tokens_per_expert, float* bias, int n_experts, float rate, int zero_tokens,
+                           stm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

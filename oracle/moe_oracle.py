@@ -518,6 +518,14 @@ def moe_layer(
     return out * routed_scaling_factor, ids, weights, aux
 
 
+def update_router_balance_bias(tokens_per_expert: torch.Tensor, bias: torch.Tensor, update_rate: float) -> torch.Tensor:
+    """moe_block.py:470-478 for one layer (after the reference's all-reduces, which are identities
+    on one GPU): ``bias + sign(mean(tokens) - tokens) * rate`` in fp32."""
+    t = tokens_per_expert.float()
+    offset = t.mean(dim=-1, keepdim=True) - t
+    return bias + torch.sign(offset) * update_rate
+
+
 # --------------------------------------------------------------------------- #
 # fp8 e4m3 (OCP "fn": no inf, max 448) with 1x128 block scales.  NOT in the reference.
 # --------------------------------------------------------------------------- #

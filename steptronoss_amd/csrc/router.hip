@@ -380,6 +380,33 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_bwd_kernel(RouterA
   }
 }
 
+// Aux-loss-free load balancing: bias[e] += sign(mean(tokens) - tokens[e]) * rate, then the token
+// counters start over.  One block; the mean is the exact integer total, rounded once, over E.
+__global__ __launch_bounds__(1024) void router_bias_update_kernel(int32_t* __restrict__ tokens,
+                                                                  float* __restrict__ bias, int n_experts, float rate,
+                                                                  bool zero_tokens) {
+  __shared__ long long wave_part[1024 / kWave];
+  __shared__ float mean_s;
+  long long mine = 0;
+  for (int e = threadIdx.x; e < n_experts; e += 1024) mine += tokens[e];
+  mine = wave_sum(mine);
+  if (threadIdx.x % kWave == 0) wave_part[threadIdx.x / kWave] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    long long total = 0;
+    for (int w = 0; w < 1024 / kWave; ++w) total += wave_part[w];
+    mean_s = float(total) / float(n_experts);
+  }
+  __syncthreads();
+  const float mean = mean_s;
+  for (int e = threadIdx.x; e < n_experts; e += 1024) {
+    const float offset = mean - float(tokens[e]);
+    const float sign = offset > 0.f ? 1.f : (offset < 0.f ? -1.f : 0.f);
+    bias[e] += sign * rate;
+    if (zero_tokens) tokens[e] = 0;
+  }
+}
+
 inline int router_blocks(int64_t n_tokens) {
   const int64_t want = (n_tokens + kRouterWaves - 1) / kRouterWaves;
   return int(want < 1 ? 1 : (want > 1024 ? 1024 : want));
@@ -452,6 +479,17 @@ int stm_router_bwd(const void* logits, int logits_dtype, int64_t n_tokens, int n
   const int need = (n_experts + kWave - 1) / kWave;
   STM_ROUTER_DISPATCH(need, (router_bwd_kernel<V><<<blocks, kRouterWaves * kWave, 0, s>>>(
                                 a, ids, grad_weights, grad_aux_or_null, hist, grad_logits)));
+  return launch_status();
+}
+
+int stm_router_bias_update(int32_t* tokens_per_expert, float* bias, int n_experts, float rate, int zero_tokens,
+                           stm_stream_t stream) {
+  using namespace stm;
+  if (n_experts < 0) return STM_ERR_ARG;
+  if (n_experts == 0) return STM_OK;
+  if (!tokens_per_expert || !bias) return STM_ERR_ARG;
+  router_bias_update_kernel<<<1, 1024, 0, as_stream(stream)>>>(tokens_per_expert, bias, n_experts, rate,
+                                                               zero_tokens != 0);
   return launch_status();
 }
 

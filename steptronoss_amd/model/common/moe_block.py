@@ -160,6 +160,7 @@ class MoEBlock(nn.Module):
         swiglu_limit=None,
         n_group=1,
         topk_group=1,
+        router_bias_update_rate=1e-3,
         device=None,
         dtype=None,
     ):
@@ -172,10 +173,18 @@ class MoEBlock(nn.Module):
         self.n_group, self.topk_group = n_group, topk_group
         self.gate = MoEGate(hidden_size, num_experts, fp32_gate_output, device=device, dtype=dtype)
         self.experts = GroupedExperts(num_experts, hidden_size, moe_hidden_size, swiglu_limit, device, dtype)
+        # aux-loss-free load balancing (reference moe_block.py:199-215): a selection-only bias per
+        # expert, the tokens each expert received since the last update, and the update rate
+        self.router_bias_update_rate = router_bias_update_rate
+        self.micro_batch_count = 0
         if aux_loss_free_balance:
             self.register_buffer("router_balance_bias", torch.zeros(num_experts, dtype=torch.float32, device=device))
+            self.register_buffer(
+                "local_tokens_per_expert", torch.zeros(num_experts, dtype=torch.int32, device=device), persistent=False
+            )
         else:
             self.router_balance_bias = None
+            self.local_tokens_per_expert = None
 
     def route(self, logits):
         return forward_router(
@@ -193,8 +202,35 @@ class MoEBlock(nn.Module):
         x2 = x.reshape(-1, shape[-1])
         if logits is None:
             logits = self.gate(x2)
-        ids, weights, aux, _hist = self.route(logits)
+        ids, weights, aux, hist = self.route(logits)
+        if self.local_tokens_per_expert is not None and self.training:
+            with torch.no_grad():  # reference moe_block.py:283-290
+                self.local_tokens_per_expert += hist.to(self.local_tokens_per_expert.dtype)
+                self.micro_batch_count += 1
         out = self.experts(x2, ids, weights)
         out = out.reshape(shape)
         out = bind_aux_loss(out, aux * self.aux_loss_coef)
         return out * self.routed_scaling_factor
+
+    @staticmethod
+    def update_router_balance_bias_per_gbs(models: torch.nn.Module) -> None:
+        """Once per global batch, over the whole model: every MoE layer that balances without an
+        aux loss moves its selection bias one ``router_bias_update_rate`` towards the mean load,
+        ``bias += sign(mean(tokens) - tokens) * rate``, and restarts its token count
+        (reference moe_block.py:442-491; its all-reduces over the expert / data parallel groups
+        are identities on one GPU)."""
+        from steptronoss_amd._lib import call, ptr, require_gpu, stream
+
+        for layer in models.modules():
+            if not isinstance(layer, MoEBlock) or layer.router_balance_bias is None or layer.micro_batch_count <= 0:
+                continue
+            bias, tokens = layer.router_balance_bias, layer.local_tokens_per_expert
+            if bias.dtype != torch.float32:  # the bias lives in fp32 whatever the model's dtype (:423-432)
+                layer.router_balance_bias = bias = bias.float()
+            dev = require_gpu(bias, tokens)
+            with torch.cuda.device(dev):
+                call(
+                    "stm_router_bias_update", ptr(tokens), ptr(bias), bias.numel(), float(layer.router_bias_update_rate),
+                    1, stream(),
+                )  # fmt: skip
+            layer.micro_batch_count = 0

@@ -271,3 +271,39 @@ def test_nothing_routed_early_out_matches_reference_when_validating():
         assert float(out.abs().sum()) == 0.0  # no read-back: nothing to combine
     finally:
         M.settings.validate_fused = old
+
+
+def test_balance_bias_update_matches_oracle():
+    from steptronoss_amd._lib import call, ptr, stream
+
+    gen = torch.Generator().manual_seed(5)
+    for E in (4, 128, 1500):
+        tokens = torch.randint(0, 3000, (E,), generator=gen, dtype=torch.int32)
+        tokens[:2] = int(tokens.float().mean())  # some experts sit near / at the mean
+        bias = torch.randn(E, generator=gen)
+        ref = O.update_router_balance_bias(tokens, bias, 1e-3)
+        t_dev, b_dev = tokens.to(DEV), bias.to(DEV)
+        call("stm_router_bias_update", ptr(t_dev), ptr(b_dev), E, 1e-3, 1, stream())
+        assert torch.equal(b_dev.cpu(), ref)
+        assert int(t_dev.abs().sum()) == 0
+
+
+def test_moe_block_tracks_tokens_and_updates_its_bias():
+    torch.manual_seed(0)
+    blk = B.MoEBlock(64, 32, 8, 2, aux_loss_free_balance=True, router_bias_update_rate=0.01, device=DEV, dtype=torch.bfloat16)
+    blk.train()
+    x = torch.randn(48, 64, device=DEV, dtype=torch.bfloat16)
+    logits = torch.randn(48, 8, device=DEV)
+    for _ in range(3):
+        blk(x, logits)
+    assert blk.micro_batch_count == 3
+    counts = blk.local_tokens_per_expert.clone()
+    assert int(counts.sum()) == 3 * 48 * 2
+    expect = O.update_router_balance_bias(counts.cpu(), blk.router_balance_bias.cpu().clone(), 0.01)
+    B.MoEBlock.update_router_balance_bias_per_gbs(blk)
+    assert torch.equal(blk.router_balance_bias.cpu(), expect)
+    assert blk.micro_batch_count == 0 and int(blk.local_tokens_per_expert.sum()) == 0
+    # the bias steers the selection only: weights still come from the unbiased scores
+    ids, w, _aux, _hist = blk.route(logits)
+    ref_ids, ref_w, _ = O.forward_router(logits.cpu(), 2, balance_bias=expect)[:3]
+    assert torch.equal(ids.cpu(), ref_ids) and torch.allclose(w.cpu(), ref_w, atol=1e-6)

@@ -288,3 +288,13 @@ def test_te_permute_index_roundtrip_and_chunks():
     assert torch.equal(got, torch.cat([inp[3:6], inp[0:2], inp[2:3]]))
     got, gp = O.moe_sort_chunks_by_index(inp, torch.tensor([2, 1, 3]), torch.tensor([2, 0, 1]), probs=torch.arange(6.0))
     assert gp.tolist() == [3.0, 4.0, 5.0, 0.0, 1.0, 2.0]
+
+
+# ----- aux-loss-free balance bias: reference moe_block.py:470-478 -----------------------------
+def test_balance_bias_update_closed_form():
+    tokens = torch.tensor([10, 0, 5, 5])  # mean 5: over, under, at the mean twice
+    bias = torch.tensor([0.5, -0.25, 0.0, 1.0])
+    out = O.update_router_balance_bias(tokens, bias, 0.125)
+    assert torch.equal(out, torch.tensor([0.375, -0.125, 0.0, 1.0]))
+    # the update never changes the sum when loads are symmetric about the mean
+    assert float(O.update_router_balance_bias(torch.tensor([3, 1]), torch.zeros(2), 1.0).sum()) == 0.0
