@@ -129,6 +129,19 @@ int stm_unpermute_bwd(const void* grad_out, const void* in, const void* pos, int
                       int weight_dtype, void* grad_in, void* grad_weight, int64_t n_tokens, int top_k,
                       int64_t hidden, int64_t n_in_rows, int dtype, uint8_t* written_or_null, stm_stream_t stream);
 
+/* The combine with the tail of the layer folded in (MoEBlock.forward's "* routed_scaling_factor",
+ * moe_block.py:419, and MoeShareExpertFFN's "+ share_output", moe_share_expert_ffn.py:56-76):
+ *   out[t,:] = round(round(combined[t,:]) * scale) + addend[t,:]      (scale / addend optional)
+ * rounded to the row dtype after each step, i.e. bit-identical to the separate element-wise ops;
+ * and its backward, which scales (and rounds) d out before using it.  d addend = d out. */
+int stm_unpermute_fwd_epilogue(const void* in, const void* pos, int pos_is_i64, const void* weight, int weight_dtype,
+                               void* out, int64_t n_tokens, int top_k, int64_t hidden, int64_t n_in_rows, int dtype,
+                               int has_scale, float scale, const void* addend_or_null, stm_stream_t stream);
+int stm_unpermute_bwd_scaled(const void* grad_out, const void* in, const void* pos, int pos_is_i64, const void* weight,
+                             int weight_dtype, void* grad_in, void* grad_weight, int64_t n_tokens, int top_k,
+                             int64_t hidden, int64_t n_in_rows, int dtype, uint8_t* written_or_null, int has_scale,
+                             float scale, stm_stream_t stream);
+
 /* d input / d weight of moe_weighted_gather for ANY index, including one that names an input
  * row from several slots (the reference accumulates them with index_add_, moe_utils.py:302-305;
  * its own test uses such an index, tests/test_moe_utils.py:61-101).  Contributions to a row are

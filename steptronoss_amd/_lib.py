@@ -46,6 +46,8 @@ SIGNATURES = {
     "stm_permute_bwd": (I, [P, P, I, P, L, I, L, L, I, P]),
     "stm_unpermute_fwd": (I, [P, P, I, P, I, P, L, I, L, L, I, P]),
     "stm_unpermute_bwd": (I, [P, P, P, I, P, I, P, P, L, I, L, L, I, P, P]),
+    "stm_unpermute_fwd_epilogue": (I, [P, P, I, P, I, P, L, I, L, L, I, I, F, P, P]),
+    "stm_unpermute_bwd_scaled": (I, [P, P, P, I, P, I, P, P, L, I, L, L, I, P, I, F, P]),
     "stm_unpermute_bwd_general_workspace_bytes": (Z, [L, L]),
     "stm_unpermute_bwd_general": (I, [P, P, P, I, P, I, P, P, L, I, L, L, I, P, Z, P]),
     "stm_sort_by_key_workspace_bytes": (Z, [L, L]),

@@ -148,7 +148,8 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_fwd_kernel(const T* __r
                                                                     const void* __restrict__ pos,
                                                                     const void* __restrict__ weight, int wdtype,
                                                                     T* __restrict__ out, int top_k, int64_t hidden,
-                                                                    int64_t n_rows) {
+                                                                    int64_t n_rows, bool has_scale, float scale,
+                                                                    const T* __restrict__ addend) {
   using P = Pack<T, VEC>;
   const int64_t t = blockIdx.x;
   const int64_t units = hidden / VEC;
@@ -177,9 +178,23 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_fwd_kernel(const T* __r
         }
       }
     }
+    // optional tail: (combined * scale) + addend[t], each step rounded to T as separate
+    // element-wise kernels would round it
     P o;
+    if (has_scale || addend) {
+      P add{};
+      if (addend) add = reinterpret_cast<const P*>(addend + t * hidden)[u];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) o.v[j] = from_float<T>(acc[j]);
+      for (int j = 0; j < VEC; ++j) {
+        float v = round_through<T>(acc[j]);
+        if (has_scale) v = round_through<T>(v * scale);
+        if (addend) v += to_float(add.v[j]);
+        o.v[j] = from_float<T>(v);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o.v[j] = from_float<T>(acc[j]);
+    }
     reinterpret_cast<P*>(out + t * hidden)[u] = o;
   }
 }
@@ -193,7 +208,7 @@ template <typename T, int VEC, bool I64>
 __global__ __launch_bounds__(kRowThreads) void unpermute_bwd_kernel(
     const T* __restrict__ go, const T* __restrict__ in, const void* __restrict__ pos, const void* __restrict__ weight,
     int wdtype, T* __restrict__ gin, void* __restrict__ gw, int top_k, int64_t hidden, int64_t n_rows,
-    uint8_t* __restrict__ written) {
+    uint8_t* __restrict__ written, bool has_scale, float scale) {
   using P = Pack<T, VEC>;
   __shared__ float partial[kRowThreads / kWave][kDotChunk];
   const int64_t t = blockIdx.x;
@@ -206,7 +221,11 @@ __global__ __launch_bounds__(kRowThreads) void unpermute_bwd_kernel(
 #pragma unroll
     for (int c = 0; c < kDotChunk; ++c) dot[c] = 0.f;
     for (int64_t u = threadIdx.x; u < units; u += kRowThreads) {
-      const P g = reinterpret_cast<const P*>(go + t * hidden)[u];
+      P g = reinterpret_cast<const P*>(go + t * hidden)[u];
+      if (has_scale) {  // the gradient of (combined * scale): d out * scale, rounded to T
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) g.v[j] = from_float<T>(to_float(g.v[j]) * scale);
+      }
       int64_t row[kBatch];
       bool ok[kBatch];
       load_batch<I64>(pos, slot0, k0, top_k, n_rows, row, ok);
@@ -410,14 +429,17 @@ int dispatch_permute_bwd(const void* go, const void* pos, int pos_is_i64, void* 
 
 template <typename T>
 int dispatch_unpermute_fwd(const void* in, const void* pos, int pos_is_i64, const void* w, int wdtype, void* out,
-                           int64_t n_tokens, int top_k, int64_t hidden, int64_t n_rows, hipStream_t s) {
+                           int64_t n_tokens, int top_k, int64_t hidden, int64_t n_rows, bool has_scale, float scale,
+                           const void* addend, hipStream_t s) {
   const T* i = static_cast<const T*>(in);
+  const T* add = static_cast<const T*>(addend);
   T* o = static_cast<T*>(out);
   const unsigned grid = unsigned(n_tokens);
-  const bool vec = can_vectorise<T>(hidden, {in, out});
+  const bool vec = can_vectorise<T>(hidden, {in, out, addend ? addend : out});
   const bool fp32w = wdtype == STM_F32;
 #define STM_LAUNCH(VEC, I64, F32W) \
-  unpermute_fwd_kernel<T, VEC, I64, F32W><<<grid, kRowThreads, 0, s>>>(i, pos, w, wdtype, o, top_k, hidden, n_rows)
+  unpermute_fwd_kernel<T, VEC, I64, F32W><<<grid, kRowThreads, 0, s>>>(i, pos, w, wdtype, o, top_k, hidden, n_rows, \
+                                                                       has_scale, scale, add)
 #define STM_PICK(VEC)                                                        \
   if (pos_is_i64) {                                                          \
     if (fp32w) STM_LAUNCH(VEC, true, true); else STM_LAUNCH(VEC, true, false);   \
@@ -437,7 +459,7 @@ int dispatch_unpermute_fwd(const void* in, const void* pos, int pos_is_i64, cons
 template <typename T>
 int dispatch_unpermute_bwd(const void* go, const void* in, const void* pos, int pos_is_i64, const void* w, int wdtype,
                            void* gin, void* gw, int64_t n_tokens, int top_k, int64_t hidden, int64_t n_rows,
-                           uint8_t* written, hipStream_t s) {
+                           uint8_t* written, bool has_scale, float scale, hipStream_t s) {
   const T* g = static_cast<const T*>(go);
   const T* i = static_cast<const T*>(in);
   T* o = static_cast<T*>(gin);
@@ -445,7 +467,7 @@ int dispatch_unpermute_bwd(const void* go, const void* in, const void* pos, int 
   const bool vec = can_vectorise<T>(hidden, {go, in, gin});
 #define STM_LAUNCH(VEC, I64)                                                                                      \
   unpermute_bwd_kernel<T, VEC, I64><<<grid, kRowThreads, 0, s>>>(g, i, pos, w, wdtype, o, gw, top_k, hidden, n_rows, \
-                                                                 written)
+                                                                 written, has_scale, scale)
   if (vec) {
     if (pos_is_i64) STM_LAUNCH(wide_vec<T>(), true); else STM_LAUNCH(wide_vec<T>(), false);
   } else {
@@ -554,19 +576,46 @@ int stm_permute_bwd(const void* grad_out, const void* pos, int pos_is_i64, void*
   }
 }
 
-int stm_unpermute_fwd(const void* in, const void* pos, int pos_is_i64, const void* weight, int weight_dtype, void* out,
-                      int64_t n_tokens, int top_k, int64_t hidden, int64_t n_in_rows, int dtype,
-                      stm_stream_t stream) {
+int stm_unpermute_fwd_epilogue(const void* in, const void* pos, int pos_is_i64, const void* weight, int weight_dtype,
+                               void* out, int64_t n_tokens, int top_k, int64_t hidden, int64_t n_in_rows, int dtype,
+                               int has_scale, float scale, const void* addend_or_null, stm_stream_t stream) {
   using namespace stm;
   if (bad_rows(n_tokens, top_k, hidden) || n_in_rows < 0) return STM_ERR_ARG;
   if (weight_dtype < STM_F32 || weight_dtype > STM_BF16) return STM_ERR_UNSUPPORTED;
   if (n_tokens == 0 || hidden == 0) return STM_OK;
   if (!out || (top_k > 0 && (!pos || !weight)) || (n_in_rows > 0 && !in)) return STM_ERR_ARG;
   hipStream_t s = as_stream(stream);
+  const bool hs = has_scale != 0;
   switch (dtype) {
-    case STM_F32: return dispatch_unpermute_fwd<float>(in, pos, pos_is_i64, weight, weight_dtype, out, n_tokens, top_k, hidden, n_in_rows, s);
-    case STM_F16: return dispatch_unpermute_fwd<f16_t>(in, pos, pos_is_i64, weight, weight_dtype, out, n_tokens, top_k, hidden, n_in_rows, s);
-    case STM_BF16: return dispatch_unpermute_fwd<bf16_t>(in, pos, pos_is_i64, weight, weight_dtype, out, n_tokens, top_k, hidden, n_in_rows, s);
+    case STM_F32: return dispatch_unpermute_fwd<float>(in, pos, pos_is_i64, weight, weight_dtype, out, n_tokens, top_k, hidden, n_in_rows, hs, scale, addend_or_null, s);
+    case STM_F16: return dispatch_unpermute_fwd<f16_t>(in, pos, pos_is_i64, weight, weight_dtype, out, n_tokens, top_k, hidden, n_in_rows, hs, scale, addend_or_null, s);
+    case STM_BF16: return dispatch_unpermute_fwd<bf16_t>(in, pos, pos_is_i64, weight, weight_dtype, out, n_tokens, top_k, hidden, n_in_rows, hs, scale, addend_or_null, s);
+    default: return STM_ERR_UNSUPPORTED;
+  }
+}
+
+int stm_unpermute_fwd(const void* in, const void* pos, int pos_is_i64, const void* weight, int weight_dtype, void* out,
+                      int64_t n_tokens, int top_k, int64_t hidden, int64_t n_in_rows, int dtype,
+                      stm_stream_t stream) {
+  return stm_unpermute_fwd_epilogue(in, pos, pos_is_i64, weight, weight_dtype, out, n_tokens, top_k, hidden, n_in_rows,
+                                    dtype, 0, 1.f, nullptr, stream);
+}
+
+int stm_unpermute_bwd_scaled(const void* grad_out, const void* in, const void* pos, int pos_is_i64, const void* weight,
+                             int weight_dtype, void* grad_in, void* grad_weight, int64_t n_tokens, int top_k,
+                             int64_t hidden, int64_t n_in_rows, int dtype, uint8_t* written_or_null, int has_scale,
+                             float scale, stm_stream_t stream) {
+  using namespace stm;
+  if (bad_rows(n_tokens, top_k, hidden) || n_in_rows < 0) return STM_ERR_ARG;
+  if (weight_dtype < STM_F32 || weight_dtype > STM_BF16) return STM_ERR_UNSUPPORTED;
+  if (n_tokens == 0 || top_k == 0) return STM_OK;
+  if (!grad_out || !pos || !weight || !grad_weight || (n_in_rows > 0 && (!in || !grad_in))) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  const bool hs = has_scale != 0;
+  switch (dtype) {
+    case STM_F32: return dispatch_unpermute_bwd<float>(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k, hidden, n_in_rows, written_or_null, hs, scale, s);
+    case STM_F16: return dispatch_unpermute_bwd<f16_t>(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k, hidden, n_in_rows, written_or_null, hs, scale, s);
+    case STM_BF16: return dispatch_unpermute_bwd<bf16_t>(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k, hidden, n_in_rows, written_or_null, hs, scale, s);
     default: return STM_ERR_UNSUPPORTED;
   }
 }
@@ -574,18 +623,8 @@ int stm_unpermute_fwd(const void* in, const void* pos, int pos_is_i64, const voi
 int stm_unpermute_bwd(const void* grad_out, const void* in, const void* pos, int pos_is_i64, const void* weight,
                       int weight_dtype, void* grad_in, void* grad_weight, int64_t n_tokens, int top_k, int64_t hidden,
                       int64_t n_in_rows, int dtype, uint8_t* written_or_null, stm_stream_t stream) {
-  using namespace stm;
-  if (bad_rows(n_tokens, top_k, hidden) || n_in_rows < 0) return STM_ERR_ARG;
-  if (weight_dtype < STM_F32 || weight_dtype > STM_BF16) return STM_ERR_UNSUPPORTED;
-  if (n_tokens == 0 || top_k == 0) return STM_OK;
-  if (!grad_out || !pos || !weight || !grad_weight || (n_in_rows > 0 && (!in || !grad_in))) return STM_ERR_ARG;
-  hipStream_t s = as_stream(stream);
-  switch (dtype) {
-    case STM_F32: return dispatch_unpermute_bwd<float>(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k, hidden, n_in_rows, written_or_null, s);
-    case STM_F16: return dispatch_unpermute_bwd<f16_t>(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k, hidden, n_in_rows, written_or_null, s);
-    case STM_BF16: return dispatch_unpermute_bwd<bf16_t>(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens, top_k, hidden, n_in_rows, written_or_null, s);
-    default: return STM_ERR_UNSUPPORTED;
-  }
+  return stm_unpermute_bwd_scaled(grad_out, in, pos, pos_is_i64, weight, weight_dtype, grad_in, grad_weight, n_tokens,
+                                  top_k, hidden, n_in_rows, dtype, written_or_null, 0, 1.f, stream);
 }
 
 size_t stm_unpermute_bwd_general_workspace_bytes(int64_t n_slots, int64_t n_in_rows) {

@@ -136,8 +136,13 @@ class GroupedExperts(nn.Module):
         self.w1 = nn.Parameter(torch.empty(num_experts, 2 * moe_hidden_size, hidden_size, device=device, dtype=dtype))
         self.w2 = nn.Parameter(torch.empty(num_experts, hidden_size, moe_hidden_size, device=device, dtype=dtype))
 
-    def forward(self, x, token_expert_ids, token_weights):
-        return routed_grouped_ffn(self.w1, self.w2, self.activation, x, token_expert_ids, token_weights)
+    def forward(self, x, token_expert_ids, token_weights, out_scale=None, out_addend=None):
+        if out_scale is None and out_addend is None:  # the reference's call, whatever backend is selected
+            return routed_grouped_ffn(self.w1, self.w2, self.activation, x, token_expert_ids, token_weights)
+        return routed_grouped_ffn(
+            self.w1, self.w2, self.activation, x, token_expert_ids, token_weights, out_scale=out_scale,
+            out_addend=out_addend,
+        )  # fmt: skip
 
 
 class MoEBlock(nn.Module):
@@ -197,7 +202,10 @@ class MoEBlock(nn.Module):
             topk_group=self.topk_group,
         )
 
-    def forward(self, x: torch.Tensor, logits: torch.Tensor | None = None):
+    def forward(self, x: torch.Tensor, logits: torch.Tensor | None = None, shared_out: torch.Tensor | None = None):
+        """``routed(x) * routed_scaling_factor`` with the load-balance loss bound to it (reference
+        moe_block.py:376-420); with ``shared_out`` (a shared expert's output for the same tokens)
+        the sum of both, the scaling and the addition done by the combine kernel."""
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
         if logits is None:
@@ -207,10 +215,11 @@ class MoEBlock(nn.Module):
             with torch.no_grad():  # reference moe_block.py:283-290
                 self.local_tokens_per_expert += hist.to(self.local_tokens_per_expert.dtype)
                 self.micro_batch_count += 1
-        out = self.experts(x2, ids, weights)
+        scale = None if self.routed_scaling_factor == 1.0 else float(self.routed_scaling_factor)
+        addend = None if shared_out is None else shared_out.reshape(-1, shape[-1])
+        out = self.experts(x2, ids, weights, out_scale=scale, out_addend=addend)
         out = out.reshape(shape)
-        out = bind_aux_loss(out, aux * self.aux_loss_coef)
-        return out * self.routed_scaling_factor
+        return bind_aux_loss(out, aux * self.aux_loss_coef)
 
     @staticmethod
     def update_router_balance_bias_per_gbs(models: torch.nn.Module) -> None:

@@ -1,0 +1,44 @@
+"""MoE layer with an optional shared expert: ``moe(x) + share_expert(x)``.
+
+Mirror of ``MoeShareExpertFFN`` (reference steptronoss/model/common/moe_share_expert_ffn.py:27-76)
+for the part that touches the hot path: the routed experts' output, its scaling and the sum with
+the shared expert's output leave the combine kernel in one pass over ``[T, H]``.
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from steptronoss_amd.model.common.feed_forward import swiglu
+from steptronoss_amd.model.common.moe_block import MoEBlock
+
+
+class SharedExpert(nn.Module):
+    """The dense SwiGLU FFN every token goes through: ``w2(swiglu(w1(x)))`` with ``w1`` producing
+    gate and up halves (reference feed_forward.py:20-26 and the FeedForward built at
+    moe_share_expert_ffn.py:50-54).  Plain ``torch.matmul``: a dense GEMM, outside the routed path."""
+
+    def __init__(self, hidden_size: int, ffn_hidden_size: int, swiglu_limit=None, device=None, dtype=None):
+        super().__init__()
+        self.w1 = nn.Parameter(torch.empty(2 * ffn_hidden_size, hidden_size, device=device, dtype=dtype))
+        self.w2 = nn.Parameter(torch.empty(hidden_size, ffn_hidden_size, device=device, dtype=dtype))
+        nn.init.normal_(self.w1, std=0.02)
+        nn.init.normal_(self.w2, std=0.02)
+        self.swiglu_limit = swiglu_limit
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return swiglu(x @ self.w1.t(), swiglu_limit=self.swiglu_limit) @ self.w2.t()
+
+
+class MoeShareExpertFFN(nn.Module):
+    def __init__(self, moe: MoEBlock, share_expert: nn.Module | None = None):
+        super().__init__()
+        self.moe = moe
+        self.share_expert = share_expert
+        self.enable_share_expert = share_expert is not None
+
+    def forward(self, x: torch.Tensor, logits: torch.Tensor | None = None) -> torch.Tensor:
+        if not self.enable_share_expert:
+            return self.moe(x, logits)
+        return self.moe(x, logits, shared_out=self.share_expert(x))

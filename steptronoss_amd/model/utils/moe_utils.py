@@ -238,24 +238,28 @@ def hip_moe_scatter(input: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------------- unpermute
-def _combine_rows(inp: torch.Tensor, pos: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+def _combine_rows(inp: torch.Tensor, pos: torch.Tensor, weight: torch.Tensor, scale=None, addend=None) -> torch.Tensor:
+    """``out[t] = sum_k weight[t,k] * inp[pos[t,k]]``, optionally ``* scale`` and ``+ addend[t]``
+    (each step rounded to the row dtype, as separate element-wise ops would)."""
     T, K = pos.shape
     hidden = inp.shape[-1]
     out = torch.empty((T, hidden), device=inp.device, dtype=inp.dtype)
     call(
-        "stm_unpermute_fwd", ptr(inp), ptr(pos), is_i64(pos), ptr(weight), dtype_code(weight.dtype), ptr(out), T, K,
-        hidden, inp.shape[0], dtype_code(inp.dtype), stream(),
+        "stm_unpermute_fwd_epilogue", ptr(inp), ptr(pos), is_i64(pos), ptr(weight), dtype_code(weight.dtype), ptr(out),
+        T, K, hidden, inp.shape[0], dtype_code(inp.dtype), int(scale is not None), float(scale or 0.0), ptr(addend),
+        stream(),
     )  # fmt: skip
     return out
 
 
-def _combine_rows_bwd(grad_out, inp, pos, weight, grad_in, written):
+def _combine_rows_bwd(grad_out, inp, pos, weight, grad_in, written, scale=None):
     T, K = pos.shape
     hidden = inp.shape[-1]
     gw = torch.empty((T, K), device=inp.device, dtype=weight.dtype)
     call(
-        "stm_unpermute_bwd", ptr(grad_out), ptr(inp), ptr(pos), is_i64(pos), ptr(weight), dtype_code(weight.dtype),
-        ptr(grad_in), ptr(gw), T, K, hidden, inp.shape[0], dtype_code(inp.dtype), ptr(written), stream(),
+        "stm_unpermute_bwd_scaled", ptr(grad_out), ptr(inp), ptr(pos), is_i64(pos), ptr(weight),
+        dtype_code(weight.dtype), ptr(grad_in), ptr(gw), T, K, hidden, inp.shape[0], dtype_code(inp.dtype), ptr(written),
+        int(scale is not None), float(scale or 0.0), stream(),
     )  # fmt: skip
     return gw
 
@@ -539,7 +543,7 @@ class _FusedRoutedFFN(torch.autograd.Function):
     used slots are ever touched."""
 
     @staticmethod
-    def forward(ctx, w1, w2, x, token_expert_ids, token_weights, swiglu_limit):
+    def forward(ctx, w1, w2, x, token_expert_ids, token_weights, swiglu_limit, out_scale=None, out_addend=None):
         from steptronoss_amd.model.common.feed_forward import swiglu_fwd_rows
 
         dev = x.device
@@ -561,9 +565,11 @@ class _FusedRoutedFFN(torch.autograd.Function):
                 gu = _gemm_rows(xp, w1, offsets, two_f, True)
                 h = swiglu_fwd_rows(gu, swiglu_limit, live)
             y = _gemm_rows(h, w2, offsets, H, True)
-            out = _combine_rows(y, pos, token_weights)
+            addend = None if out_addend is None else out_addend.contiguous()
+            out = _combine_rows(y, pos, token_weights, out_scale, addend)
         ctx.save_for_backward(w1, w2, xp, gu, h, y, pos, offsets, token_weights)
         ctx.limit = swiglu_limit
+        ctx.out_scale = out_scale
         ctx.shape = (T, H, K, E)
         return out
 
@@ -574,13 +580,13 @@ class _FusedRoutedFFN(torch.autograd.Function):
         w1, w2, xp, gu, h, y, pos, offsets, token_weights = ctx.saved_tensors
         T, H, K, E = ctx.shape
         dev = grad_out.device
-        need_w1, need_w2, need_x, _, need_tw, _ = ctx.needs_input_grad
+        need_w1, need_w2, need_x, _, need_tw, _, _, need_addend = ctx.needs_input_grad
         gw1 = gw2 = gx = gtw = None
         with torch.cuda.device(dev):
             live = offsets[E:]
             go = grad_out.contiguous()
             gy = torch.empty_like(y)
-            gtw = _combine_rows_bwd(go, y, pos, token_weights, gy, None)
+            gtw = _combine_rows_bwd(go, y, pos, token_weights, gy, None, ctx.out_scale)
             if need_w2:
                 gw2 = _gemm_wgrad(gy, h, offsets, E)
             if need_w1 or need_x:
@@ -593,7 +599,7 @@ class _FusedRoutedFFN(torch.autograd.Function):
                 if need_x:
                     dxp = _gemm_rows(dgu, w1, offsets, H, False)
                     gx = _permute_rows_bwd(dxp, pos, H)
-        return gw1, gw2, gx, None, (gtw if need_tw else None), None
+        return gw1, gw2, gx, None, (gtw if need_tw else None), None, None, (grad_out if need_addend else None)
 
 
 _ACT_CACHE: dict = {}
@@ -642,8 +648,13 @@ def _swiglu_limit_of(act, ffn2: int, dtype, device):
     return ok, (limit if ok else None)
 
 
-def hip_routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights):
+def hip_routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights, *, out_scale=None, out_addend=None):
     """The routed expert FFN: ``combine(GEMM(act(GEMM(permute(x), w1^T)), w2^T))``.
+
+    ``out_scale`` / ``out_addend`` (not in the reference's signature, default off) fold the tail
+    of the layer into the combine: ``out * out_scale + out_addend`` with the roundings of the
+    separate ops (``* routed_scaling_factor``, reference moe_block.py:419; ``+ share_output``,
+    moe_share_expert_ffn.py:56-76).
 
     Drop-in for ``routed_grouped_ffn`` (reference moe_utils.py:222-244), differentiable in
     ``w1``, ``w2``, ``x`` and ``token_weights``.  ``w1`` is ``[E, 2F, H]``, ``w2`` ``[E, H, F]``.
@@ -666,23 +677,28 @@ def hip_routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights):
     ids = token_expert_ids.contiguous()
     tw = token_weights.contiguous()
     with torch.cuda.device(dev):
+        def tail(out):  # the unfused form of the optional tail
+            if out_scale is not None:
+                out = out * out_scale
+            return out if out_addend is None else out + out_addend
+
         if settings.validate_fused and not bool((ids >= 0).any()):
             # The reference reads the routed count back on the host and, when it is zero, returns
             # x * sum(weights) (moe_utils.py:230-232).  Only the validating mode pays for that
             # read-back; without it an all-unrouted batch gives zeros (nothing to combine).
-            return x * token_weights.sum()
+            return tail(x * token_weights.sum())
         fused, limit = _swiglu_limit_of(act, w1.shape[1], x.dtype, dev)
         if fused:
-            return _FusedRoutedFFN.apply(w1c, w2c, xc, ids, tw, limit)
+            return _FusedRoutedFFN.apply(w1c, w2c, xc, ids, tw, limit, out_scale, out_addend)
         _hist, offsets, pos, _status = route_plan(ids, E)
         n_rows = T * K
         rows = _no_sync_permute(xc, pos, n_rows)
         rows = _GroupedGemm.apply(rows, w1c, offsets, n_rows, True)
         rows = act(rows)
         rows = _GroupedGemm.apply(rows.contiguous(), w2c, offsets, n_rows, True)
-        return _CombineInjective.apply(rows, pos, tw)
+        return tail(_CombineInjective.apply(rows, pos, tw))
 
 
 @optimizable(alternatives={BACKEND_NAME: hip_routed_grouped_ffn, "fused": hip_routed_grouped_ffn})
-def routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights):
-    return hip_routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights)
+def routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights, **tail):
+    return hip_routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights, **tail)

@@ -307,3 +307,53 @@ def test_moe_block_tracks_tokens_and_updates_its_bias():
     ids, w, _aux, _hist = blk.route(logits)
     ref_ids, ref_w, _ = O.forward_router(logits.cpu(), 2, balance_bias=expect)[:3]
     assert torch.equal(ids.cpu(), ref_ids) and torch.allclose(w.cpu(), ref_w, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_combine_tail_matches_the_separate_ops_bit_for_bit(dtype):
+    gen = torch.Generator().manual_seed(8)
+    T, K, H, E = 96, 4, 128, 8
+    ids = make_topk_ids(T, K, E, gen=gen, invalid_frac=0.1).to(DEV)
+    pos = M.index_compute(ids, M.histogram(ids, E))
+    n_rows = int((ids >= 0).sum())
+    rows = torch.randn(n_rows, H, generator=gen).to(dtype).to(DEV)
+    w = torch.rand(T, K, generator=gen).to(DEV)
+    shared = torch.randn(T, H, generator=gen).to(dtype).to(DEV)
+    plain = M._combine_rows(rows, pos, w)
+    assert torch.equal(M._combine_rows(rows, pos, w, 2.5, None), plain * 2.5)
+    assert torch.equal(M._combine_rows(rows, pos, w, None, shared), plain + shared)
+    assert torch.equal(M._combine_rows(rows, pos, w, 2.5, shared), plain * 2.5 + shared)
+    go = torch.randn(T, H, generator=gen).to(dtype).to(DEV)
+    g_ref, g_fused = torch.empty_like(rows), torch.empty_like(rows)
+    gw_ref = M._combine_rows_bwd((go * 2.5).contiguous(), rows, pos, w, g_ref, None)
+    gw_fused = M._combine_rows_bwd(go, rows, pos, w, g_fused, None, 2.5)
+    assert torch.equal(g_ref, g_fused) and torch.equal(gw_ref, gw_fused)
+
+
+def test_shared_expert_layer_matches_the_unfused_composition():
+    from steptronoss_amd.model.common.moe_share_expert_ffn import MoeShareExpertFFN, SharedExpert
+
+    torch.manual_seed(1)
+    H, F, E, K, T = 64, 48, 8, 2, 80
+    moe = B.MoEBlock(H, F, E, K, aux_loss_coef=0.01, routed_scaling_factor=2.5, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():  # like the reference, the expert weights come uninitialised
+        moe.experts.w1.normal_(std=0.1)
+        moe.experts.w2.normal_(std=0.1)
+    layer = MoeShareExpertFFN(moe, SharedExpert(H, 32, device=DEV, dtype=torch.bfloat16))
+    x = torch.randn(T, H, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    logits = torch.randn(T, E, device=DEV)
+    out = layer(x, logits)
+    go = torch.randn_like(out)
+    out.backward(go)
+    fused = [x.grad.clone()] + [p.grad.clone() for p in layer.parameters() if p.grad is not None]
+    x.grad = None
+    for p in layer.parameters():
+        p.grad = None
+    # the reference's composition: moe(x) (scaled inside) + share_expert(x) as separate ops
+    ref = moe(x, logits) + layer.share_expert(x)
+    ref.backward(go)
+    unfused = [x.grad.clone()] + [p.grad.clone() for p in layer.parameters() if p.grad is not None]
+    assert torch.equal(out, ref)
+    assert len(fused) == len(unfused)
+    for a, b in zip(fused, unfused):
+        assert rel_l2(a, b.float()) <= 1e-2  # same roundings except where autograd sums two gradient paths
