@@ -220,6 +220,14 @@ int stm_grouped_gemm_dswiglu(const void* grad_y, const void* w2, const void* gat
 int stm_grouped_gemm_wgrad(const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
                            int64_t m_cap, int p, int q, int dtype, stm_stream_t stream);
 
+/* The same product ADDED to an fp32 buffer accum [G, p, q] instead of stored in the operands'
+ * dtype: the weight gradient accumulated straight into the optimizer's fp32 "main_grad"
+ * (the reference adds param.grad into it afterwards, optimizer/base_gradient_manager.py:153-155),
+ * which saves writing and re-reading the 16-bit gradient.  STM_ERR_UNSUPPORTED for shapes the
+ * 256 x 256 kernels do not take (p or q below 256 or not a multiple of 8, fp32 operands). */
+int stm_grouped_gemm_wgrad_accum(const void* x, const void* y, float* accum, const int32_t* offsets, int n_groups,
+                                 int64_t m_cap, int p, int q, int dtype, stm_stream_t stream);
+
 /* ------------------------------------------------------------------------------------
  * SwiGLU between the two expert GEMMs.
  * ---------------------------------------------------------------------------------- */

@@ -58,6 +58,7 @@ SIGNATURES = {
     "stm_gemm_workspace_bytes": (Z, [L, I]),
     "stm_grouped_gemm": (I, [P, P, P, P, I, L, I, I, I, I, P, Z, P]),
     "stm_grouped_gemm_wgrad": (I, [P, P, P, P, I, L, I, I, I, P]),
+    "stm_grouped_gemm_wgrad_accum": (I, [P, P, P, P, I, L, I, I, I, P]),
     "stm_grouped_gemm_swiglu": (I, [P, P, P, P, P, I, L, I, I, I, F, I, P, Z, P]),
     "stm_grouped_gemm_dswiglu": (I, [P, P, P, P, P, I, L, I, I, I, F, I, P, Z, P]),
     "stm_quantize_e4m3_1x128": (I, [P, I, L, L, P, P, P]),

@@ -13,7 +13,7 @@ namespace stm {
 int launch_mfma_rows(int dtype, const void* a, const void* b, void* c, const int32_t* offsets, int n_groups,
                      int64_t m_cap, int n, int k, int b_is_nk, void* ws, size_t ws_bytes, hipStream_t s);
 int launch_mfma_wgrad(int dtype, const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
-                      int64_t m_cap, int p, int q, hipStream_t s);
+                      int64_t m_cap, int p, int q, int accumulate, hipStream_t s);
 
 namespace {
 
@@ -263,6 +263,16 @@ int stm_grouped_gemm_dswiglu(const void* grad_y, const void* w2, const void* gat
   return launch_dma_swiglu_bwd(dtype, p, offsets, n_groups, m_cap, workspace, as_stream(stream));
 }
 
+int stm_grouped_gemm_wgrad_accum(const void* x, const void* y, float* accum, const int32_t* offsets, int n_groups,
+                                 int64_t m_cap, int p_dim, int q_dim, int dtype, stm_stream_t stream) {
+  using namespace stm;
+  if (n_groups < 0 || m_cap < 0 || p_dim < 0 || q_dim < 0) return STM_ERR_ARG;
+  if ((dtype != STM_BF16 && dtype != STM_F16) || n_groups > kMaxGroups) return STM_ERR_UNSUPPORTED;
+  if (n_groups == 0 || p_dim == 0 || q_dim == 0) return STM_OK;
+  if (!accum || !offsets || (m_cap > 0 && (!x || !y))) return STM_ERR_ARG;
+  return launch_mfma_wgrad(dtype, x, y, accum, offsets, n_groups, m_cap, p_dim, q_dim, 1, as_stream(stream));
+}
+
 int stm_grouped_gemm_wgrad(const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
                            int64_t m_cap, int p_dim, int q_dim, int dtype, stm_stream_t stream) {
   using namespace stm;
@@ -271,7 +281,7 @@ int stm_grouped_gemm_wgrad(const void* x, const void* y, void* out, const int32_
   if (n_groups == 0 || p_dim == 0 || q_dim == 0) return STM_OK;
   if (!out || !offsets || (m_cap > 0 && (!x || !y))) return STM_ERR_ARG;
   hipStream_t s = as_stream(stream);
-  const int fast = launch_mfma_wgrad(dtype, x, y, out, offsets, n_groups, m_cap, p_dim, q_dim, s);
+  const int fast = launch_mfma_wgrad(dtype, x, y, out, offsets, n_groups, m_cap, p_dim, q_dim, 0, s);
   if (fast != STM_ERR_UNSUPPORTED) return fast;
   GenericArgs p{};
   p.a = x;

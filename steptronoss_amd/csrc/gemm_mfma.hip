@@ -19,7 +19,7 @@ namespace stm {
 
 int launch_dma_rows(int dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap, int b_is_nk,
                     void* ws, hipStream_t s);
-int launch_dma_wgrad(int dtype, const GemmArgs& base, int n_groups, int64_t m_cap, hipStream_t s);
+int launch_dma_wgrad(int dtype, const GemmArgs& base, int n_groups, int64_t m_cap, int accumulate, hipStream_t s);
 
 namespace {
 
@@ -335,8 +335,9 @@ int launch_mfma_rows(int dtype, const void* a, const void* b, void* c, const int
                            : rows_typed<f16_t>(p, offsets, n_groups, m_cap, b_is_nk, ws, s);
 }
 
+// accumulate != 0: `out` is an fp32 buffer the product is added to (only the 256 x 256 kernels do that).
 int launch_mfma_wgrad(int dtype, const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
-                      int64_t m_cap, int p_dim, int q_dim, hipStream_t s) {
+                      int64_t m_cap, int p_dim, int q_dim, int accumulate, hipStream_t s) {
   (void)m_cap;
   if (dtype != STM_BF16 && dtype != STM_F16) return STM_ERR_UNSUPPORTED;
   if (p_dim % 8 != 0 || q_dim % 8 != 0) return STM_ERR_UNSUPPORTED;
@@ -354,9 +355,10 @@ int launch_mfma_wgrad(int dtype, const void* x, const void* y, void* out, const 
   p.n_j = q_dim;
   p.n_groups = n_groups;
   if (p_dim >= 256 && q_dim >= 256) {
-    const int st = launch_dma_wgrad(dtype, p, n_groups, m_cap, s);
+    const int st = launch_dma_wgrad(dtype, p, n_groups, m_cap, accumulate, s);
     if (st != STM_ERR_UNSUPPORTED) return st;
   }
+  if (accumulate) return STM_ERR_UNSUPPORTED;
   return dtype == STM_BF16 ? wgrad_typed<bf16_t>(p, n_groups, s) : wgrad_typed<f16_t>(p, n_groups, s);
 }
 

@@ -202,7 +202,7 @@ struct TileState {
 };
 
 // What the epilogue does with the accumulators.
-enum Epilogue { kStore = 0, kSwigluFwd = 1, kSwigluBwd = 2 };
+enum Epilogue { kStore = 0, kSwigluFwd = 1, kSwigluBwd = 2, kAccumF32 = 3 };
 
 // WAVES = 4: one wave per SIMD, 2 x 2 waves of 128 x 128 outputs each.
 // WAVES = 8: two waves per SIMD, 4 x 2 waves of 64 x 128 outputs each: while one wave of a SIMD
@@ -218,10 +218,14 @@ enum Epilogue { kStore = 0, kSwigluFwd = 1, kSwigluBwd = 2 };
 //   beside it, both rounded as the unfused kernels round them.
 // EPI = kSwigluBwd (d h = d y * W2): d h is never stored; the epilogue reads gate_up and stores
 //   d gate_up.
+// EPI = kAccumF32 (wgrad): the product is added to an fp32 buffer of the output's shape (a
+//   gradient accumulator) instead of being stored in T.
 template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int kBK, int EPI>
 __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs p) {
   static_assert(kBK == 64 || kBK == 32, "contraction elements per stage");
-  static_assert(EPI == kStore || (WAVES == 8 && !WGRAD && !A_KM), "fused epilogues: rows form, 8 waves");
+  static_assert(EPI == kStore || EPI == kAccumF32 || (WAVES == 8 && !WGRAD && !A_KM),
+                "fused SwiGLU epilogues: rows form, 8 waves");
+  static_assert(EPI != kAccumF32 || (WAVES == 8 && WGRAD), "accumulation into an fp32 buffer: wgrad, 8 waves");
   static_assert(EPI != kSwigluFwd || !B_KM, "the fused forward reads W1 rows K-contiguous");
   constexpr int kStages = (1 << kStagesBytesLog2) / ((BM + BN) * kBK * 2);
   constexpr int WROWS = WAVES / 2;                   // wave rows; two wave columns
@@ -307,7 +311,10 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       t.valid_i = p.n_i - i0;
       a += lo * p.lda + i0;
       b += lo * p.ldb + j0;
-      c += g * p.c_group + int64_t(i0) * p.ldc + j0;
+      if constexpr (EPI == kAccumF32)
+        c = reinterpret_cast<T*>(static_cast<float*>(p.c) + g * p.c_group + int64_t(i0) * p.ldc + j0);
+      else
+        c += g * p.c_group + int64_t(i0) * p.ldc + j0;
       // contraction rows past the end of the group are past the end of the buffer: zeros
       const int64_t ab = int64_t(n_k) * p.lda * 2 - int64_t(i0) * 2;
       const int64_t bb = int64_t(n_k) * p.ldb * 2 - int64_t(j0) * 2;
@@ -517,7 +524,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     // by the bounds check; lanes past the column bound aim past the end of any descriptor.  (No
     // lane-dependent branch: the tile bookkeeping stays provably wave-uniform around it.)
     constexpr uint32_t kDroppedOffset = 0xffffff00u;
-    const uint32_t row_bytes_c = uint32_t(p.ldc) * 2u;
+    const uint32_t row_bytes_c = uint32_t(p.ldc) * (EPI == kAccumF32 ? 4u : 2u);
     const int live_rows = cur.valid_i < BM ? cur.valid_i : BM;
     const __amdgpu_buffer_rsrc_t rsrc_c =
         __builtin_amdgcn_make_buffer_rsrc(static_cast<void*>(cur.c), 0, int(uint32_t(live_rows) * row_bytes_c), 0x00020000);
@@ -572,7 +579,40 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
         const int row = it * 8 + rd_row;
         return *reinterpret_cast<const uint4*>(buf + row * 128 + ((rd_c ^ ((row >> 1) & 7)) * 16));
       };
-      if constexpr (EPI == kStore) {
+      if constexpr (EPI == kAccumF32) {
+        // 32 columns of fp32 at a time (rows of 128 bytes in the scratch, as above): read the
+        // accumulator buffer, add, write back
+        unsigned char* wr32 = buf + r * 128;
+#pragma unroll
+        for (int i = 0; i < ATM; ++i) {
+          const int row0 = (WROWS * i + wave_row) * 32;
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              *reinterpret_cast<float4*>(wr32 + (((q * 2 + tl / 32) ^ ((r >> 1) & 7)) * 16)) =
+                  make_float4(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+            const int col = wave_j + j * 32 + rd_c * 4;
+            const bool col_live = col < valid_j;
+            float4 old[4];
+#pragma unroll
+            for (int it = 0; it < 4; ++it)
+              old[it] = __builtin_bit_cast(
+                  float4, __builtin_amdgcn_raw_buffer_load_b128(
+                              rsrc_c,
+                              col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes_c + uint32_t(col) * 4u : kDroppedOffset,
+                              0, 0));
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+              const float4 v = __builtin_bit_cast(float4, staged(it));
+              const float4 sum = make_float4(old[it].x + v.x, old[it].y + v.y, old[it].z + v.z, old[it].w + v.w);
+              __builtin_amdgcn_raw_buffer_store_b128(
+                  __builtin_bit_cast(u32x4_t, sum), rsrc_c,
+                  col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes_c + uint32_t(col) * 4u : kDroppedOffset, 0, 0);
+            }
+          }
+        }
+      } else if constexpr (EPI == kStore) {
 #pragma unroll
         for (int i = 0; i < ATM; ++i) {
           const int row0 = (WROWS * i + wave_row) * 32;
@@ -818,13 +858,19 @@ int launch_dma_swiglu_bwd(int dtype, const GemmArgs& base, const int32_t* offset
   return launch<f16_t, kDmaBM, kDmaBN, false, true, false, 32, kSwigluBwd>(p, s);
 }
 
-int launch_dma_wgrad(int dtype, const GemmArgs& base, int n_groups, int64_t m_cap, hipStream_t s) {
+// accumulate != 0: base.c is an fp32 buffer [G, P, Q] and the product is added to it.
+int launch_dma_wgrad(int dtype, const GemmArgs& base, int n_groups, int64_t m_cap, int accumulate, hipStream_t s) {
   GemmArgs p = base;
   if (p.n_i % 8 != 0 || p.n_j % 8 != 0) return STM_ERR_UNSUPPORTED;
   if (m_cap * p.lda * 2 >= (int64_t(1) << 32) || m_cap * p.ldb * 2 >= (int64_t(1) << 32)) return STM_ERR_UNSUPPORTED;
+  if (int64_t(kDmaBM) * p.ldc * 4 >= (int64_t(1) << 32)) return STM_ERR_UNSUPPORTED;
   p.tiles_i = (p.n_i + kDmaBM - 1) / kDmaBM;
   p.tiles_j = (p.n_j + kDmaBN - 1) / kDmaBN;
   p.n_groups = n_groups;
+  if (accumulate) {
+    if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, true, true, true, 32, kAccumF32>(p, s);
+    return launch<f16_t, kDmaBM, kDmaBN, true, true, true, 32, kAccumF32>(p, s);
+  }
   if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, true, true, true, 32>(p, s);
   return launch<f16_t, kDmaBM, kDmaBN, true, true, true, 32>(p, s);
 }

@@ -41,10 +41,16 @@ class Settings:
         ``validate_fused`` is set; with it the op also reproduces the reference's early-out
         for a batch in which no slot is routed (``x * token_weights.sum()``), which needs the
         routed count on the host.
+    fuse_main_grad: a weight of ``routed_grouped_ffn`` that carries an fp32 ``main_grad``
+        buffer (the gradient manager's accumulator, reference
+        optimizer/base_gradient_manager.py:153-155) gets its gradient added straight into that
+        buffer by the wgrad kernel; autograd then sees ``None`` for it, so no 16-bit gradient
+        is written, re-read and added afterwards.
     """
 
     validate: bool = True
     validate_fused: bool = False
+    fuse_main_grad: bool = False
 
 
 settings = Settings()
@@ -537,6 +543,21 @@ def _gemm_dswiglu_rows(gy: torch.Tensor, w2: torch.Tensor, gu: torch.Tensor, off
     return dgu if ok else None
 
 
+def _wgrad_into_main_grad(x: torch.Tensor, y: torch.Tensor, offsets: torch.Tensor, weight: torch.Tensor) -> bool:
+    """``weight.main_grad[g] += x[rows of g]^T @ y[rows of g]`` when the switch is on, the
+    buffer is there (fp32, the weight's shape) and the kernel takes the shape."""
+    main_grad = getattr(weight, "main_grad", None)
+    if not settings.fuse_main_grad or main_grad is None:
+        return False
+    if main_grad.dtype != torch.float32 or main_grad.shape != weight.shape or not main_grad.is_contiguous():
+        return False
+    n_groups, p, q = weight.shape
+    return try_call(
+        "stm_grouped_gemm_wgrad_accum", ptr(x), ptr(y), ptr(main_grad), ptr(offsets), n_groups, x.shape[0], p, q,
+        dtype_code(x.dtype), stream(),
+    )  # fmt: skip
+
+
 class _FusedRoutedFFN(torch.autograd.Function):
     """route_plan -> permute -> GEMM(w1^T) -> SwiGLU -> GEMM(w2^T) -> combine in one autograd
     node: no host round trip, intermediates are sized for all ``T*K`` slots and only the rows of
@@ -587,14 +608,14 @@ class _FusedRoutedFFN(torch.autograd.Function):
             go = grad_out.contiguous()
             gy = torch.empty_like(y)
             gtw = _combine_rows_bwd(go, y, pos, token_weights, gy, None, ctx.out_scale)
-            if need_w2:
+            if need_w2 and not _wgrad_into_main_grad(gy, h, offsets, w2):
                 gw2 = _gemm_wgrad(gy, h, offsets, E)
             if need_w1 or need_x:
                 dgu = _gemm_dswiglu_rows(gy, w2, gu, offsets, ctx.limit)
                 if dgu is None:
                     dh = _gemm_rows(gy, w2, offsets, h.shape[1], False)
                     dgu = swiglu_bwd_rows(gu, dh, ctx.limit, live)
-                if need_w1:
+                if need_w1 and not _wgrad_into_main_grad(dgu, xp, offsets, w1):
                     gw1 = _gemm_wgrad(dgu, xp, offsets, E)
                 if need_x:
                     dxp = _gemm_rows(dgu, w1, offsets, H, False)

@@ -142,3 +142,54 @@ def test_fused_swiglu_declines_small_or_odd_shapes():
     w1 = torch.randn(2, 48, 40, device=dev).bfloat16()
     offsets = M._group_offsets(torch.tensor([30, 34]), dev)
     assert M._gemm_swiglu_rows(a, w1, offsets, None) == (None, None)  # fewer than 4096 rows, k % 32 != 0
+
+
+# ----- wgrad added straight into an fp32 accumulator -------------------------------------------
+def test_wgrad_accumulates_into_fp32_buffer():
+    gen = torch.Generator().manual_seed(4)
+    sizes = [700, 0, 1300, 33]
+    m, E, P, Q = sum(sizes), len(sizes), 256, 384
+    x = torch.randn(m, P, generator=gen).bfloat16().to(DEV)
+    y = torch.randn(m, Q, generator=gen).bfloat16().to(DEV)
+    offsets = M._group_offsets(torch.tensor(sizes), torch.device(DEV))
+    accum = torch.randn(E, P, Q, generator=gen).to(DEV)
+    before = accum.clone()
+    from steptronoss_amd._lib import dtype_code, ptr, stream, try_call
+
+    ok = try_call("stm_grouped_gemm_wgrad_accum", ptr(x), ptr(y), ptr(accum), ptr(offsets), E, m, P, Q,
+                  dtype_code(x.dtype), stream())  # fmt: skip
+    assert ok
+    _, ref = O.grouped_gemm_grads(x.cpu().float(), torch.zeros(E, P, Q), torch.tensor(sizes), False, y.cpu().float())
+    assert rel_l2(accum - before, ref) <= 1e-5  # fp32 all the way: no 16-bit rounding of the gradient
+    assert torch.equal(accum[1], before[1])  # the empty group adds nothing
+    # a second call keeps adding
+    try_call("stm_grouped_gemm_wgrad_accum", ptr(x), ptr(y), ptr(accum), ptr(offsets), E, m, P, Q,
+             dtype_code(x.dtype), stream())  # fmt: skip
+    assert rel_l2(accum - before, 2 * ref) <= 1e-5
+
+
+def test_routed_ffn_can_accumulate_weight_grads_into_main_grad():
+    from steptronoss_amd.model.common.feed_forward import swiglu
+
+    gen = torch.Generator().manual_seed(6)
+    T, H, E, K, F = 1024, 256, 4, 4, 256
+    x = torch.randn(T, H, generator=gen).bfloat16().to(DEV)
+    w1 = (torch.randn(E, 2 * F, H, generator=gen) * 0.05).bfloat16().to(DEV).requires_grad_(True)
+    w2 = (torch.randn(E, H, F, generator=gen) * 0.05).bfloat16().to(DEV).requires_grad_(True)
+    ids = torch.stack([torch.randperm(E, generator=gen)[:K] for _ in range(T)]).to(DEV)
+    tw = torch.rand(T, K, generator=gen).to(DEV)
+    go = torch.randn(T, H, generator=gen).bfloat16().to(DEV)
+    M.routed_grouped_ffn(w1, w2, swiglu, x, ids, tw).backward(go)
+    g1, g2 = w1.grad.clone(), w2.grad.clone()
+    w1.grad = w2.grad = None
+    w1.main_grad = torch.ones(w1.shape, device=DEV)
+    w2.main_grad = torch.ones(w2.shape, device=DEV)
+    old = M.settings.fuse_main_grad
+    try:
+        M.settings.fuse_main_grad = True
+        M.routed_grouped_ffn(w1, w2, swiglu, x, ids, tw).backward(go)
+    finally:
+        M.settings.fuse_main_grad = old
+    assert w1.grad is None and w2.grad is None  # nothing left for autograd to add
+    assert rel_l2(w1.main_grad - 1, g1.float()) <= 1e-2
+    assert rel_l2(w2.main_grad - 1, g2.float()) <= 1e-2
