@@ -38,7 +38,7 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 # from hardware counters collected in separate profiler runs of this script (FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB copies of
 # --traffic-probe); the summaries of those runs are kept under profiles/.  None = not measured.
-MEASURED_GEMM_TRAFFIC_BYTES = {"c2": 2.445e9, "c3": None, "c4": None}
+MEASURED_GEMM_TRAFFIC_BYTES = {"c2": 2.455e9, "c3": None, "c4": None}
 
 WORKLOADS = {
     "c2": dict(T=16384, H=2048, E=128, K=8, F=768, sigmoid=False, norm=True, n_group=1, topk_group=1, std=0.02),
@@ -183,7 +183,7 @@ def main():
     achieved = flops_per_launch / (avg_launch_ms * 1e-3) / 1e12 if gemm_calls else 0.0
     roofline = {
         "bound": "mfma",
-        "kernel": "persistent_gemm_kernel (grouped GEMM fwd / dgrad / wgrad, 256x256x64 tiles)",
+        "kernel": "persistent_gemm_kernel (grouped GEMM fwd / dgrad / wgrad, 256x256 tiles, SwiGLU in two epilogues)",
         "achieved": achieved,
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
@@ -194,9 +194,9 @@ def main():
         "launches_per_step": gemm_calls / args.steps,
     }
 
-    def bw(name, nbytes):
-        t = timing.get(name)
-        if not t or not t["calls"]:
+    def bw(names, nbytes):
+        t = next((timing[n] for n in names.split("|") if n in timing and timing[n]["calls"]), None)
+        if t is None:
             return None
         gbps = nbytes / (t["avg_us"] * 1e-6) / 1e9
         return {"GB/s": gbps, "avg_us": t["avg_us"], "bytes": nbytes, "frac_of_hbm_peak": gbps / PEAK_HBM_GBPS}
@@ -204,8 +204,8 @@ def main():
     bandwidth = {
         "permute_fwd": bw("stm_permute_fwd", T * H * e + N * H * e + 4 * N),
         "permute_bwd": bw("stm_permute_bwd", N * H * e + T * H * e + 4 * N),
-        "unpermute_fwd": bw("stm_unpermute_fwd", N * H * e + T * H * e + 8 * N),
-        "unpermute_bwd": bw("stm_unpermute_bwd", T * H * e + 2 * N * H * e + 12 * N),
+        "unpermute_fwd": bw("stm_unpermute_fwd_epilogue|stm_unpermute_fwd", N * H * e + T * H * e + 8 * N),
+        "unpermute_bwd": bw("stm_unpermute_bwd_scaled|stm_unpermute_bwd", T * H * e + 2 * N * H * e + 12 * N),
         "route_plan_us": timing.get("stm_route_plan", {}).get("avg_us"),
         "router_fwd_us": timing.get("stm_router_fwd", {}).get("avg_us"),
         "router_bwd_us": timing.get("stm_router_bwd", {}).get("avg_us"),
