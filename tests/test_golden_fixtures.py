@@ -1,0 +1,113 @@
+"""The reference's own known-answer vectors (tests/golden/reference_kats.json) against the
+oracle (CPU) and against the HIP path through the C ABI (GPU)."""
+
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+
+with open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")) as fh:
+    G = json.load(fh)
+
+
+def _backends():
+    yield pytest.param("oracle", id="oracle")
+    yield pytest.param("hip", id="hip", marks=pytest.mark.gpu)
+
+
+def _ops(which):
+    if which == "oracle":
+        return O, "cpu", O
+    from steptronoss_amd.model.utils import moe_utils as M
+    from steptronoss_amd.model.utils import permute_utils as P
+
+    return M, "cuda:0", P
+
+
+@pytest.mark.parametrize("which", _backends())
+def test_histogram_and_index_compute(which):
+    ops, dev, _ = _ops(which)
+    for c in G["histogram"]:
+        out = ops.histogram(torch.tensor(c["ids"], dtype=torch.int64, device=dev), c["experts"])
+        assert out.dtype == torch.int32 and out.tolist() == c["expect"], c["source"]
+    for c in G["histogram_errors"]:
+        with pytest.raises((ValueError, AssertionError), match=c["match"]):
+            ops.histogram(torch.tensor(c["ids"], dtype=torch.int64, device=dev), c["experts"])
+    for c in G["index_compute"]:
+        out = ops.index_compute(torch.tensor(c["ids"], device=dev), torch.tensor(c["hist"], dtype=torch.int32, device=dev))
+        assert out.dtype == torch.int32 and out.tolist() == c["expect"], c["source"]
+    for c in G["index_compute_errors"]:
+        with pytest.raises(AssertionError, match=c["match"]):
+            ops.index_compute(torch.tensor(c["ids"], device=dev), torch.tensor(c["hist"], dtype=torch.int32, device=dev))
+
+
+@pytest.mark.parametrize("which", _backends())
+def test_gather_and_scatter_values_and_gradients(which):
+    ops, dev, _ = _ops(which)
+    for c in G["moe_weighted_gather"]:
+        x = torch.tensor(c["x"], device=dev, requires_grad=True)
+        w = torch.tensor(c["w"], device=dev, requires_grad=True)
+        out = ops.moe_weighted_gather(x, torch.tensor(c["idx"], device=dev), w)
+        assert torch.allclose(out.detach().cpu(), torch.tensor(c["expect"])), c["source"]
+        out.sum().backward()
+        assert torch.allclose(x.grad.cpu(), torch.tensor(c["grad_x_of_sum"])), c["source"]
+        assert torch.allclose(w.grad.cpu(), torch.tensor(c["grad_w_of_sum"])), c["source"]
+    for c in G["moe_scatter"]:
+        x = torch.tensor(c["x"], device=dev, requires_grad=True)
+        out = ops.moe_scatter(x, torch.tensor(c["idx"], device=dev))
+        assert torch.equal(out.detach().cpu(), torch.tensor(c["expect"])), c["source"]
+        out.sum().backward()
+        assert torch.equal(x.grad.cpu(), torch.tensor(c["grad_x_of_sum"])), c["source"]
+    for c in G["scatter_gather_symmetry"]:
+        x = torch.tensor(c["x"], device=dev)
+        idx = torch.tensor(c["idx"], device=dev)
+        back = ops.moe_weighted_gather(ops.moe_scatter(x, idx), idx, torch.ones(idx.shape, device=dev))
+        assert torch.allclose(back, x * (idx >= 0).sum(1, keepdim=True)), c["source"]
+
+
+@pytest.mark.parametrize("which", _backends())
+def test_grouped_gemm_reference_shapes(which):
+    ops, dev, _ = _ops(which)
+    for c in G["grouped_gemm_shapes"]:
+        for trans_b in c["trans_b"]:
+            gen = torch.Generator().manual_seed(0)
+            sizes = torch.tensor(c["batch_sizes"])
+            a = torch.randn(int(sizes.sum()), c["k"], generator=gen)
+            b = torch.randn(len(c["batch_sizes"]), *((c["n"], c["k"]) if trans_b else (c["k"], c["n"])), generator=gen)
+            expect, row = [], 0
+            for g, m in enumerate(c["batch_sizes"]):  # the reference test's per-group matmul
+                expect.append(a[row : row + m] @ (b[g].t() if trans_b else b[g]))
+                row += m
+            out = ops.grouped_gemm(a.to(dev), b.to(dev), sizes, trans_b=trans_b)
+            assert torch.allclose(out.cpu(), torch.cat(expect), rtol=1e-2, atol=1e-2), c["source"]
+
+
+@pytest.mark.parametrize("which", _backends())
+def test_te_style_helpers(which):
+    _, dev, P = _ops(which)
+    c = G["te_permute"]
+    tokens = torch.tensor(c["tokens"], device=dev)
+    mask = torch.tensor(c["mask"], dtype=torch.bool, device=dev)
+    probs = torch.tensor(c["mask_probs"], device=dev)
+    if P is O:
+        out, rid, pp = P.moe_permute(tokens, mask, probs=probs)
+    else:
+        out, pp, rid = P.moe_permute_with_probs(tokens, probs, mask)
+    assert rid.tolist() == c["mask_expect_row_ids"]
+    assert torch.equal(out.cpu(), torch.tensor(c["tokens"])[c["mask_expect_tokens"]])
+    assert torch.equal(pp.cpu(), torch.tensor(c["mask_probs"]).t().reshape(-1)[c["mask_expect_row_ids"]])
+    back = P.moe_unpermute(out, rid, merging_probs=probs, restore_shape=tokens.shape, map_type="mask")
+    assert torch.allclose(back.cpu(), torch.tensor(c["tokens"]))
+    rm = torch.tensor(c["index_map"], device=dev)
+    out, rid = P.moe_permute(tokens, rm, map_type="index")
+    assert rid.tolist() == c["index_expect_row_ids"]
+    iprobs = torch.tensor(c["index_probs"], device=dev)
+    back = P.moe_unpermute(out, rid, merging_probs=iprobs, restore_shape=tokens.shape, map_type="index")
+    assert torch.allclose(back.cpu(), torch.tensor(c["tokens"]))
+    ch = c["chunks"]
+    inp = torch.arange(2 * ch["rows"], dtype=torch.float32, device=dev).view(ch["rows"], 2)
+    got = P.moe_sort_chunks_by_index(inp, torch.tensor(ch["split_sizes"]), torch.tensor(ch["sorted_index"]))
+    assert torch.equal(got.cpu(), inp.cpu()[ch["expect_row_order"]])
