@@ -53,21 +53,70 @@ __device__ __forceinline__ uint64_t lanemask_lt() {
   return l == 0 ? 0ull : (~0ull >> (64 - l));
 }
 
-template <typename T>
-__device__ __forceinline__ T wave_sum(T v) {
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-  return v;
+// ---- wave-wide reductions of 32-bit values on the DPP path (row shifts inside the 16-lane rows,
+// then two row broadcasts; the total arrives in lane 63 and is handed to every lane through a
+// scalar register).  An order of magnitude less latency than six dependent LDS-crossbar
+// shuffles, which is what the routing kernels are made of.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_move(int keep, int src) {
+  return __builtin_amdgcn_update_dpp(keep, src, CTRL, ROW_MASK, 0xf, false);
+}
+
+template <typename T, typename Op>
+__device__ __forceinline__ T wave_reduce_dpp(T v, T identity, Op op) {
+  static_assert(sizeof(T) == 4, "32-bit values");
+  const int id = __builtin_bit_cast(int, identity);
+#define STM_DPP_STEP(CTRL, MASK) v = op(v, __builtin_bit_cast(T, dpp_move<CTRL, MASK>(id, __builtin_bit_cast(int, v))))
+  STM_DPP_STEP(0x111, 0xf);  // row_shr:1
+  STM_DPP_STEP(0x112, 0xf);  // row_shr:2
+  STM_DPP_STEP(0x114, 0xf);  // row_shr:4
+  STM_DPP_STEP(0x118, 0xf);  // row_shr:8   -> lane 15 of every row holds the row's total
+  STM_DPP_STEP(0x142, 0xa);  // row_bcast:15 into rows 1 and 3
+  STM_DPP_STEP(0x143, 0xc);  // row_bcast:31 into rows 2 and 3 -> lane 63 holds the total
+#undef STM_DPP_STEP
+  return __builtin_bit_cast(T, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 template <typename T>
-__device__ __forceinline__ T wave_max(T v) {
+__device__ __forceinline__ T wave_sum(T v) {
+  if constexpr (sizeof(T) == 4) {
+    return wave_reduce_dpp(v, T(0), [](T a, T b) { return a + b; });
+  } else {
 #pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) {
-    T o = __shfl_xor(v, off, kWave);
-    v = o > v ? o : v;
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
   }
-  return v;
+}
+
+// (callers pass values for which the smallest representable number is a neutral element)
+__device__ __forceinline__ float wave_max(float v) {
+  return wave_reduce_dpp(v, -__builtin_inff(), [](float a, float b) { return fmaxf(a, b); });
+}
+__device__ __forceinline__ int32_t wave_max(int32_t v) {
+  return wave_reduce_dpp(v, int32_t(0x80000000), [](int32_t a, int32_t b) { return a > b ? a : b; });
+}
+
+// (value, index) arg-max over the wave: larger value wins, equal values -> smaller index.
+__device__ __forceinline__ void wave_argmax(float& v, int& idx) {
+  const int neutral_v = __builtin_bit_cast(int, -__builtin_inff());
+#define STM_DPP_STEP(CTRL, MASK)                                                                   \
+  {                                                                                                \
+    const float ov = __builtin_bit_cast(float, dpp_move<CTRL, MASK>(neutral_v, __builtin_bit_cast(int, v))); \
+    const int oi = dpp_move<CTRL, MASK>(0x7fffffff, idx);                                          \
+    if (ov > v || (ov == v && oi < idx)) {                                                         \
+      v = ov;                                                                                      \
+      idx = oi;                                                                                    \
+    }                                                                                              \
+  }
+  STM_DPP_STEP(0x111, 0xf)
+  STM_DPP_STEP(0x112, 0xf)
+  STM_DPP_STEP(0x114, 0xf)
+  STM_DPP_STEP(0x118, 0xf)
+  STM_DPP_STEP(0x142, 0xa)
+  STM_DPP_STEP(0x143, 0xc)
+#undef STM_DPP_STEP
+  v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+  idx = __builtin_amdgcn_readlane(idx, 63);
 }
 
 // In-place exclusive scan of a[0..n) in LDS by the whole workgroup; returns the total.

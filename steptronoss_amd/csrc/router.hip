@@ -75,19 +75,6 @@ __device__ __forceinline__ void token_scores(const RouterArgs& a, int64_t t, int
   }
 }
 
-// (value, index) arg-max over the wave: larger value wins, equal values -> smaller index.
-__device__ __forceinline__ void wave_argmax(float& v, int& idx) {
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) {
-    const float ov = __shfl_xor(v, off, kWave);
-    const int oi = __shfl_xor(idx, off, kWave);
-    if (ov > v || (ov == v && oi < idx)) {
-      v = ov;
-      idx = oi;
-    }
-  }
-}
-
 template <int V>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_fwd_kernel(RouterArgs a, int64_t* __restrict__ ids,
                                                                          float* __restrict__ weights,

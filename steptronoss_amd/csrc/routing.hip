@@ -133,9 +133,16 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(int32_t* __restrict_
   const int64_t s_end = s_begin + chunk < n_segments ? s_begin + chunk : n_segments;
   if (tid < 2) flags[tid] = 0;
 
+  constexpr int kAhead = 8;  // segment counters fetched together: the loops below are latency-bound
   for (int e = el; e < n_experts; e += lanes_e) {
     int32_t sum = 0;
-    for (int64_t s = s_begin; s < s_end; ++s) sum += counts[s * n_experts + e];
+    for (int64_t s0 = s_begin; s0 < s_end; s0 += kAhead) {
+      int32_t c[kAhead];
+#pragma unroll
+      for (int j = 0; j < kAhead; ++j) c[j] = s0 + j < s_end ? counts[(s0 + j) * n_experts + e] : 0;
+#pragma unroll
+      for (int j = 0; j < kAhead; ++j) sum += c[j];
+    }
     partial[g * n_experts + e] = sum;
   }
   __syncthreads();
@@ -187,10 +194,15 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(int32_t* __restrict_
   if (!write_table) return;
   for (int e = el; e < n_experts; e += lanes_e) {
     int32_t run = base[e] + partial[g * n_experts + e];
-    for (int64_t s = s_begin; s < s_end; ++s) {
-      const int32_t c = counts[s * n_experts + e];
-      counts[s * n_experts + e] = run;
-      run += c;
+    for (int64_t s0 = s_begin; s0 < s_end; s0 += kAhead) {
+      int32_t c[kAhead];
+#pragma unroll
+      for (int j = 0; j < kAhead; ++j) c[j] = s0 + j < s_end ? counts[(s0 + j) * n_experts + e] : 0;
+#pragma unroll
+      for (int j = 0; j < kAhead; ++j) {
+        if (s0 + j < s_end) counts[(s0 + j) * n_experts + e] = run;
+        run += c[j];
+      }
     }
   }
 }
