@@ -29,7 +29,12 @@ fp8 e4m3 quantiser     PARITY UNPINNED AGAINST THE REFERENCE (it has no fp8 MoE
                        path); exhaustive 256-code decode table, round trip,
                        saturation
 TE-style permute       brute-force expectations of tests/test_permute_utils.py
+update_router_balance  closed form on a hand-worked vector (over / under / at the
+_bias                  mean), sign symmetry
 =====================  ==========================================================
+
+The reference's literal test vectors are also kept as data in
+``tests/golden/reference_kats.json`` and run against these functions.
 """
 
 from __future__ import annotations
