@@ -32,6 +32,7 @@ if ROOT not in sys.path:
 
 METRIC = "routed grouped-FFN fwd+bwd TFLOP/s + permute/unpermute GB/s, 1 MI355X"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_FP32_TFLOPS = 157.3  # MI355X dense fp32 MFMA (the fp32 toy workload)
 PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 
 # HBM bytes per grouped-GEMM launch (fetched + written, mean over the six launches of a step),
@@ -41,6 +42,7 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 MEASURED_GEMM_TRAFFIC_BYTES = {"c2": 2.455e9, "c3": None, "c4": None}
 
 WORKLOADS = {
+    "c1": dict(T=4096, H=1024, E=8, K=2, F=2048, sigmoid=False, norm=False, n_group=1, topk_group=1, std=0.02, dtype="fp32"),
     "c2": dict(T=16384, H=2048, E=128, K=8, F=768, sigmoid=False, norm=True, n_group=1, topk_group=1, std=0.02),
     "c3": dict(T=16384, H=2048, E=128, K=8, F=768, sigmoid=False, norm=True, n_group=1, topk_group=1, std=0.02, zipf=1.2),
     "c4": dict(T=8192, H=7168, E=256, K=8, F=2048, sigmoid=True, norm=True, n_group=8, topk_group=4, std=0.006),
@@ -50,7 +52,7 @@ WORKLOADS = {
 def make_inputs(cfg, seed, device):
     gen = torch.Generator(device=device).manual_seed(seed)
     T, H, E, F = cfg["T"], cfg["H"], cfg["E"], cfg["F"]
-    bf = torch.bfloat16
+    bf = torch.float32 if cfg.get("dtype") == "fp32" else torch.bfloat16
     x = (torch.randn(T, H, generator=gen, device=device) * cfg["std"]).to(bf)
     w1 = torch.empty(E, 2 * F, H, device=device, dtype=bf)
     w2 = torch.empty(E, H, F, device=device, dtype=bf)
@@ -173,7 +175,9 @@ def main():
     value = flops / (ms_per_step * 1e-3) / 1e12
 
     timing = kt.summary()
-    e = 2  # bytes per bf16 element
+    fp32 = cfg.get("dtype") == "fp32"
+    e = 4 if fp32 else 2  # bytes per element
+    peak = PEAK_FP32_TFLOPS if fp32 else PEAK_BF16_TFLOPS
     gemm_entries = ("stm_grouped_gemm", "stm_grouped_gemm_wgrad", "stm_grouped_gemm_swiglu", "stm_grouped_gemm_dswiglu")
     gemm_calls = sum(timing[n]["calls"] for n in gemm_entries if n in timing)
     gemm_ms = sum(timing[n]["total_ms"] for n in gemm_entries if n in timing)
@@ -183,11 +187,12 @@ def main():
     achieved = flops_per_launch / (avg_launch_ms * 1e-3) / 1e12 if gemm_calls else 0.0
     roofline = {
         "bound": "mfma",
-        "kernel": "persistent_gemm_kernel (grouped GEMM fwd / dgrad / wgrad, 256x256 tiles, SwiGLU in two epilogues)",
+        "kernel": "generic_gemm_kernel (fp32 FMA tiles; priced against the fp32 MFMA peak)" if fp32
+        else "persistent_gemm_kernel (grouped GEMM fwd / dgrad / wgrad, 256x256 tiles, SwiGLU in two epilogues)",
         "achieved": achieved,
-        "peak": PEAK_BF16_TFLOPS,
+        "peak": peak,
         "unit": "TFLOP/s",
-        "frac": achieved / PEAK_BF16_TFLOPS,
+        "frac": achieved / peak,
         "traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(args.workload),
         "flops_per_launch": flops_per_launch,
         "avg_launch_us": avg_launch_ms * 1e3,
@@ -225,12 +230,12 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": cfg.get("dtype", "bf16"),
         "data": "synthetic",
         "config": {
-            "workload": f"{args.workload}: MoE layer T={T} H={H} E={E} top-{K} F={F} bf16, "
+            "workload": f"{args.workload}: MoE layer T={T} H={H} E={E} top-{K} F={F} {cfg.get('dtype', 'bf16')}, "
             + ("sigmoid group-limited" if cfg["sigmoid"] else "softmax")
-            + " routing, renormalised weights; router + routed grouped FFN, fwd+bwd",
+            + " routing" + (", renormalised weights" if cfg["norm"] else "") + "; router + routed grouped FFN, fwd+bwd",
             "tokens": T,
             "hidden": H,
             "experts": E,
@@ -238,7 +243,7 @@ def main():
             "expert_ffn": F,
             "seed": args.seed,
         },
-        "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS,
+        "frac_of_mfma_peak": value / peak,
         "roofline": roofline,
         "bandwidth": bandwidth,
         "entry_avg_us": entry_us,

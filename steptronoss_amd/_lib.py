@@ -138,10 +138,10 @@ def try_call(name: str, *args) -> bool:
     hook = _call_hook
     token = hook.before(name) if hook is not None else None
     code = getattr(load(), name)(*args)
+    if code == ERR_UNSUPPORTED:
+        return False  # nothing was launched, so nothing is timed
     if hook is not None:
         hook.after(name, token)
-    if code == ERR_UNSUPPORTED:
-        return False
     if code != 0:
         raise RuntimeError(f"{name} failed: {status_string(code)} (status {code})")
     return True

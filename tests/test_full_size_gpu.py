@@ -1,4 +1,4 @@
-"""The hot path at the full sizes of the benchmark configurations (c2, c3, c4), checked through
+"""The hot path at the full sizes of the benchmark configurations (c1 fp32; c2, c3, c4 bf16), checked through
 properties that do not need an oracle run of that size: permutations are permutations, stable
 and expert-sorted; permuted rows are bit-exact copies; permute -> combine with unit weights
 multiplies by K exactly; sampled rows / experts / tokens of the GEMMs and of the whole layer
@@ -12,10 +12,14 @@ from tests.helpers import rel_l2
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
-TOL = 1e-2  # bf16 storage, fp32 accumulation
+TOL = 1e-2  # bf16 storage, fp32 accumulation; the fp32 configuration is held to 1e-4
 
 
-@pytest.fixture(scope="module", params=["c2", "c3", "c4"])
+def tol_of(case):
+    return 1e-4 if case["x"].dtype == torch.float32 else TOL
+
+
+@pytest.fixture(scope="module", params=["c1", "c2", "c3", "c4"])
 def case(request):
     from steptronoss_amd.model.common.moe_block import forward_router
 
@@ -40,7 +44,8 @@ def test_router_invariants(case):
     assert bool((srt[:, 1:] != srt[:, :-1]).all()), "an expert was picked twice for a token"
     assert torch.equal(hist.long(), torch.bincount(ids.reshape(-1), minlength=E))
     assert int(hist.sum()) == T * K
-    assert float((weights.sum(1) - 1).abs().max()) < 1e-5  # renormalised
+    if cfg["norm"]:
+        assert float((weights.sum(1) - 1).abs().max()) < 1e-5  # renormalised
     assert bool((weights[:, 1:] <= weights[:, :-1] + 1e-7).all()), "weights are not in selection order"
     if cfg["n_group"] > 1:
         groups = ids // (E // cfg["n_group"])
@@ -115,11 +120,11 @@ def test_grouped_gemm_samples_match_fp32(case):
             continue
         rows = torch.arange(lo, hi, device=DEV)[torch.linspace(0, hi - lo - 1, min(64, hi - lo)).long().to(DEV)]
         ref = xp.detach()[rows].float() @ w1[e].float().t()
-        assert rel_l2(out.detach()[rows], ref) <= TOL
+        assert rel_l2(out.detach()[rows], ref) <= tol_of(case)
         ref_da = go[rows].float() @ w1[e].float()
-        assert rel_l2(xp.grad[rows], ref_da) <= TOL
+        assert rel_l2(xp.grad[rows], ref_da) <= tol_of(case)
         ref_dw = go[lo:hi].float().t() @ xp.detach()[lo:hi].float()
-        assert rel_l2(w.grad[e], ref_dw) <= TOL
+        assert rel_l2(w.grad[e], ref_dw) <= tol_of(case)
     empty = torch.nonzero(sizes == 0).reshape(-1)
     if empty.numel():
         assert float(w.grad[empty.to(DEV)].abs().sum()) == 0.0
@@ -147,8 +152,8 @@ def test_layer_samples_match_fp32(case):
             y = (w2[e].float() @ h).to(x.dtype).float()
             acc = acc + wt[k] * y
         acc.backward(go[t].float())
-        assert rel_l2(out.detach()[t], acc.detach()) <= TOL
-        assert rel_l2(tw.grad[t], wt.grad) <= 2 * TOL
-        assert rel_l2(xg.grad[t], xt.grad) <= 2 * TOL
+        assert rel_l2(out.detach()[t], acc.detach()) <= tol_of(case)
+        assert rel_l2(tw.grad[t], wt.grad) <= 2 * tol_of(case)
+        assert rel_l2(xg.grad[t], xt.grad) <= 2 * tol_of(case)
     assert a.grad.shape == w1.shape and b.grad.shape == w2.shape
     assert bool(torch.isfinite(a.grad).all()) and bool(torch.isfinite(b.grad).all())
