@@ -207,13 +207,36 @@ int stm_grouped_gemm(const void* a, const void* b, void* c, const int32_t* offse
  * Results are bit-identical to stm_grouped_gemm followed by stm_swiglu_fwd / stm_swiglu_bwd.
  * Return STM_ERR_UNSUPPORTED for shapes the fused kernels do not take (k not a multiple of 32,
  * ffn not a multiple of 8, fewer than 4096 rows, fp32): callers then use the unfused pair.
- * Workspace as for stm_grouped_gemm. */
-int stm_grouped_gemm_swiglu(const void* a, const void* w1, void* gate_up, void* h, const int32_t* offsets, int n_groups,
-                            int64_t m_cap, int ffn, int k, int has_limit, float limit, int dtype, void* workspace,
-                            size_t workspace_bytes, stm_stream_t stream);
+ * Workspace as for stm_grouped_gemm.
+ *
+ * row_scale (fp32 [m_cap], may be NULL = all ones) moves the combine weight of a row
+ * (MoEWeightedGather, moe_utils.py:270-281: out[t] = sum_k w[t,k] * y[pos(t,k)]) in front of the
+ * second GEMM, which is linear in its rows: the forward stores h * row_scale[r]; the backward
+ * takes grad_y as the gradient of that scaled product, so d h = row_scale[r] * (grad_y * w2[g]).
+ * row_dot (fp32 [m_cap, stm_grouped_gemm_dswiglu_row_dot_parts(ffn)], may be NULL) receives
+ * partial sums of sum_f swiglu(gate_up)[r, f] * (grad_y * w2[g])[r, f], the gradient of
+ * row_scale[r] (the same number as moe_utils.py:298, grad_output . y[pos], since
+ * go . (W2 h) = (W2^T go) . h); every live row gets all its parts written. */
+int stm_grouped_gemm_swiglu(const void* a, const void* w1, void* gate_up, void* h, const float* row_scale,
+                            const int32_t* offsets, int n_groups, int64_t m_cap, int ffn, int k, int has_limit,
+                            float limit, int dtype, void* workspace, size_t workspace_bytes, stm_stream_t stream);
+int stm_grouped_gemm_dswiglu_row_dot_parts(int ffn);
 int stm_grouped_gemm_dswiglu(const void* grad_y, const void* w2, const void* gate_up, void* grad_gate_up,
-                             const int32_t* offsets, int n_groups, int64_t m_cap, int ffn, int k, int has_limit,
-                             float limit, int dtype, void* workspace, size_t workspace_bytes, stm_stream_t stream);
+                             const float* row_scale, float* row_dot, const int32_t* offsets, int n_groups,
+                             int64_t m_cap, int ffn, int k, int has_limit, float limit, int dtype, void* workspace,
+                             size_t workspace_bytes, stm_stream_t stream);
+
+/* Between slot order ([T, K], token-major) and row order (pos = index_compute's output):
+ *   stm_slot_values_to_rows: rows[pos[s]] = float(values[s]) for every slot with pos[s] >= 0
+ *                            (values: fp32/fp16/bf16 by value_dtype; rows fp32 [n_rows]);
+ *   stm_row_parts_to_slots : out[s] = sum_p parts[pos[s], p] (0 for pos[s] < 0), parts fp32
+ *                            [n_rows, n_parts], out in out_dtype.
+ * Together with row_scale / row_dot above they carry token_weights into the fused expert FFN
+ * and its gradient back (no counterpart in the reference, which weights in the combine). */
+int stm_slot_values_to_rows(const void* values, int value_dtype, const int32_t* pos, int64_t n_slots, float* rows,
+                            int64_t n_rows, stm_stream_t stream);
+int stm_row_parts_to_slots(const float* parts, int n_parts, const int32_t* pos, int64_t n_slots, int64_t n_rows,
+                           void* out, int out_dtype, stm_stream_t stream);
 
 /* grouped_gemm wgrad, function_imple.py:54-69: out[g] = x[rows of g]^T @ y[rows of g],
  * x:[m_cap, p], y:[m_cap, q], out:[G, p, q]; an empty group gives zeros (:56-58). */

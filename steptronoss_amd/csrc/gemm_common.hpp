@@ -59,6 +59,13 @@ struct GemmArgs {
   int ffn;
   int has_limit;
   float limit;
+  // Optional per-row factor of the fused epilogues (fp32 [M], null = 1): the forward writes
+  // h * row_scale; the backward takes the product as the gradient of that scaled h, i.e. uses
+  // row_scale * (d y * w2) as d h, and, when row_dot is given, also writes
+  // sum_f h[r, f] * (d y * w2)[r, f] (the gradient of row_scale[r]) as 2 * tiles_j partial sums
+  // per row: row_dot is fp32 [M, 2 * tiles_j].
+  const float* row_scale;
+  float* row_dot;
 };
 
 // Fused SwiGLU forms of the rows GEMM (gemm_mfma_dma.hip); STM_ERR_UNSUPPORTED when the shape does not fit.

@@ -227,9 +227,9 @@ int fused_args(const void* a, const void* b, void* c, void* c2, const int32_t* o
 }
 }  // namespace
 
-int stm_grouped_gemm_swiglu(const void* a, const void* w1, void* gate_up, void* h, const int32_t* offsets, int n_groups,
-                            int64_t m_cap, int ffn, int k, int has_limit, float limit, int dtype, void* workspace,
-                            size_t workspace_bytes, stm_stream_t stream) {
+int stm_grouped_gemm_swiglu(const void* a, const void* w1, void* gate_up, void* h, const float* row_scale,
+                            const int32_t* offsets, int n_groups, int64_t m_cap, int ffn, int k, int has_limit,
+                            float limit, int dtype, void* workspace, size_t workspace_bytes, stm_stream_t stream) {
   using namespace stm;
   GemmArgs p;
   const int st = fused_args(a, w1, gate_up, h, offsets, n_groups, m_cap, ffn, k, has_limit, limit, dtype, workspace,
@@ -242,12 +242,16 @@ int stm_grouped_gemm_swiglu(const void* a, const void* w1, void* gate_up, void* 
   p.b_group = 2 * int64_t(ffn) * k;
   p.n_j = 2 * ffn;
   p.n_k = k;
+  p.row_scale = row_scale;
   return launch_dma_swiglu_fwd(dtype, p, offsets, n_groups, m_cap, workspace, as_stream(stream));
 }
 
+int stm_grouped_gemm_dswiglu_row_dot_parts(int ffn) { return ffn > 0 ? 2 * ((ffn + 255) / 256) : 0; }
+
 int stm_grouped_gemm_dswiglu(const void* grad_y, const void* w2, const void* gate_up, void* grad_gate_up,
-                             const int32_t* offsets, int n_groups, int64_t m_cap, int ffn, int k, int has_limit,
-                             float limit, int dtype, void* workspace, size_t workspace_bytes, stm_stream_t stream) {
+                             const float* row_scale, float* row_dot, const int32_t* offsets, int n_groups,
+                             int64_t m_cap, int ffn, int k, int has_limit, float limit, int dtype, void* workspace,
+                             size_t workspace_bytes, stm_stream_t stream) {
   using namespace stm;
   GemmArgs p;
   const int st = fused_args(grad_y, w2, grad_gate_up, const_cast<void*>(gate_up), offsets, n_groups, m_cap, ffn, k,
@@ -260,6 +264,8 @@ int stm_grouped_gemm_dswiglu(const void* grad_y, const void* w2, const void* gat
   p.b_group = int64_t(ffn) * k;
   p.n_j = ffn;
   p.n_k = k;
+  p.row_scale = row_scale;
+  p.row_dot = row_dot;
   return launch_dma_swiglu_bwd(dtype, p, offsets, n_groups, m_cap, workspace, as_stream(stream));
 }
 

@@ -198,6 +198,7 @@ struct TileState {
   T* c2;             // second output / extra input of a fused epilogue (first row of the tile)
   uint32_t soff_b0;  // scalar offset of this wave's first B load of a stage at contraction step 0
   int col0;          // first output column of the tile (fused SwiGLU: first gate column)
+  int row0;          // rows form: first row of the tile in the whole problem
   int valid_i, valid_j, n_steps;
 };
 
@@ -298,6 +299,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     uint32_t a_bytes, b_bytes;
     t.valid_j = (EPI == kSwigluFwd ? p.ffn : p.n_j) - j0;
     t.col0 = j0;
+    t.row0 = 0;
     t.c2 = nullptr;
     t.soff_b0 = 0;
     if constexpr (WGRAD) {
@@ -327,6 +329,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       mt.rows = __builtin_amdgcn_readfirstlane(mt.rows);
       n_k = p.n_k;
       t.valid_i = mt.rows;
+      t.row0 = mt.row0;
       a += int64_t(mt.row0) * p.lda;
       c += int64_t(mt.row0) * p.ldc + (EPI == kStore ? j0 : 0);
       if constexpr (EPI != kStore) t.c2 = static_cast<T*>(p.c2) + int64_t(mt.row0) * p.ldc2;
@@ -636,6 +639,15 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
         const __amdgpu_buffer_rsrc_t rsrc_2 = __builtin_amdgcn_make_buffer_rsrc(
             static_cast<void*>(cur.c2), 0, int(uint32_t(live_rows) * row_bytes_2), 0x00020000);
         const uint32_t up_bytes = uint32_t(p.ffn) * 2u;  // from a gate column to its up column
+        // the optional per-row factor: a descriptor over the live rows of the tile
+        const bool has_scale = p.row_scale != nullptr;
+        const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(has_scale ? p.row_scale + cur.row0 : p.row_scale), 0,
+            has_scale ? int(uint32_t(live_rows) * 4u) : 0, 0x00020000);
+        auto row_scale_of = [&](int row) {  // rows past the live ones read 0; their outputs are dropped anyway
+          return has_scale ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, uint32_t(row) * 4u, 0, 0))
+                           : 1.f;
+        };
         if constexpr (EPI == kSwigluFwd) {
           // accumulator tiles 0,1 of this wave: 64 gate columns; tiles 2,3: their up columns
           const int col = cur.col0 + (wave % 2) * 64 + rd_c * 8;  // gate column = column of h
@@ -655,17 +667,32 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
             store_round(rsrc_c, row_bytes_c, 0u);
             stage([&](int jj, int q, int e) { return acc[i][2 + jj][q * 4 + e]; });
             store_round(rsrc_c, row_bytes_c, up_bytes);
+            const float scale = row_scale_of(row0 + r);  // in the accumulators a lane owns one row
             stage([&](int jj, int q, int e) {  // from the values as stored: h = swiglu(rounded gate, rounded up)
               return swiglu_value(round_to<T>(acc[i][jj][q * 4 + e]), round_to<T>(acc[i][2 + jj][q * 4 + e]), has_limit,
-                                  limit);
+                                  limit) *
+                     scale;
             });
             store_round(rsrc_2, row_bytes_2, 0u);
           }
         } else {
           // the accumulators hold d h; gate and up come from gate_up (c2), d gate | d up go to c
+          // row_dot: one partial sum per row and per 128-column half of a column tile
+          const int n_parts = 2 * p.tiles_j;
+          const bool has_dot = p.row_dot != nullptr;
+          const __amdgpu_buffer_rsrc_t rsrc_d = __builtin_amdgcn_make_buffer_rsrc(
+              has_dot ? p.row_dot + int64_t(cur.row0) * n_parts : p.row_dot, 0,
+              has_dot ? int(uint32_t(live_rows) * uint32_t(n_parts) * 4u) : 0, 0x00020000);
+          const int part = (cur.col0 / BN) * 2 + wave % 2;
 #pragma unroll
           for (int i = 0; i < ATM; ++i) {
             const int row0 = (WROWS * i + wave_row) * 32;
+            float scale[4], dot[4];
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+              scale[it] = row_scale_of(row0 + it * 8 + rd_row);
+              dot[it] = 0.f;
+            }
 #pragma unroll
             for (int round = 0; round < kColRounds; ++round) {
               const int col = cur.col0 + wave_j + round * 64 + rd_c * 8;
@@ -688,7 +715,10 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                   float dg, du;
-                  swiglu_grads(to_float(gv.v[e]), to_float(uv.v[e]), to_float(dv.v[e]), has_limit, limit, dg, du);
+                  const float g = to_float(gv.v[e]), u = to_float(uv.v[e]), d = to_float(dv.v[e]);
+                  float h_val;
+                  swiglu_grads(g, u, d * scale[it], has_limit, limit, dg, du, h_val);
+                  dot[it] += h_val * d;
                   og.v[e] = from_float<T>(dg);
                   ou.v[e] = from_float<T>(du);
                 }
@@ -698,6 +728,17 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, ou), rsrc_c,
                                                        col_live ? at + up_bytes : kDroppedOffset, 0, 0);
               }
+            }
+            // the eight lanes of a row (rd_c = 0..7) add up in the last of them, which stores
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+              float v = dot[it];
+              v += __builtin_bit_cast(float, dpp_move<0x111, 0xf>(0, __builtin_bit_cast(int, v)));  // row_shr:1
+              v += __builtin_bit_cast(float, dpp_move<0x112, 0xf>(0, __builtin_bit_cast(int, v)));  // row_shr:2
+              v += __builtin_bit_cast(float, dpp_move<0x114, 0xf>(0, __builtin_bit_cast(int, v)));  // row_shr:4
+              __builtin_amdgcn_raw_buffer_store_b32(
+                  __builtin_bit_cast(uint32_t, v), rsrc_d,
+                  rd_c == 7 ? uint32_t((row0 + it * 8 + rd_row) * n_parts + part) * 4u : kDroppedOffset, 0, 0);
             }
           }
         }

@@ -317,6 +317,30 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const V* __res
   for (int64_t u = threadIdx.x % kWave; u < units; u += kWave) out[j * units + u] = ok ? x[i * units + u] : zero;
 }
 
+// ---------------------------------------------------------------- slot order <-> row order
+// rows[pos[s]] = values[s] for the slots that name a row.
+template <typename W>
+__global__ void slot_values_to_rows_kernel(const W* __restrict__ values, const int32_t* __restrict__ pos,
+                                           int64_t n_slots, float* __restrict__ rows, int64_t n_rows) {
+  const int64_t s = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (s >= n_slots) return;
+  const int64_t r = pos[s];
+  if (r >= 0 && r < n_rows) rows[r] = to_float(values[s]);
+}
+
+// out[s] = sum of the n_parts numbers of row pos[s].
+template <typename W>
+__global__ void row_parts_to_slots_kernel(const float* __restrict__ parts, int n_parts, const int32_t* __restrict__ pos,
+                                          int64_t n_slots, int64_t n_rows, W* __restrict__ out) {
+  const int64_t s = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (s >= n_slots) return;
+  const int64_t r = pos[s];
+  float sum = 0.f;
+  if (r >= 0 && r < n_rows)
+    for (int q = 0; q < n_parts; ++q) sum += parts[r * n_parts + q];
+  out[s] = from_float<W>(sum);
+}
+
 // ---------------------------------------------------------------- index check
 template <bool I64>
 __global__ void claim_rows_kernel(const void* __restrict__ pos, int64_t n_slots, int64_t n_rows,
@@ -719,6 +743,40 @@ int stm_index_check(const void* pos, int pos_is_i64, int64_t n_slots, int64_t n_
     summarize_pos_kernel<false><<<1, 1024, 0, s>>>(pos, n_slots, status);
     claim_rows_kernel<false><<<grid, 256, 0, s>>>(pos, n_slots, n_rows, owner, status);
     verify_rows_kernel<false><<<grid, 256, 0, s>>>(pos, n_slots, n_rows, owner, status);
+  }
+  return launch_status();
+}
+
+int stm_slot_values_to_rows(const void* values, int value_dtype, const int32_t* pos, int64_t n_slots, float* rows,
+                            int64_t n_rows, stm_stream_t stream) {
+  using namespace stm;
+  if (n_slots < 0 || n_rows < 0) return STM_ERR_ARG;
+  if (n_slots == 0 || n_rows == 0) return STM_OK;
+  if (!values || !pos || !rows) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  const unsigned grid = unsigned((n_slots + 255) / 256);
+  switch (value_dtype) {
+    case STM_F32: slot_values_to_rows_kernel<<<grid, 256, 0, s>>>(static_cast<const float*>(values), pos, n_slots, rows, n_rows); break;
+    case STM_F16: slot_values_to_rows_kernel<<<grid, 256, 0, s>>>(static_cast<const f16_t*>(values), pos, n_slots, rows, n_rows); break;
+    case STM_BF16: slot_values_to_rows_kernel<<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(values), pos, n_slots, rows, n_rows); break;
+    default: return STM_ERR_UNSUPPORTED;
+  }
+  return launch_status();
+}
+
+int stm_row_parts_to_slots(const float* parts, int n_parts, const int32_t* pos, int64_t n_slots, int64_t n_rows,
+                           void* out, int out_dtype, stm_stream_t stream) {
+  using namespace stm;
+  if (n_slots < 0 || n_rows < 0 || n_parts < 0) return STM_ERR_ARG;
+  if (n_slots == 0) return STM_OK;
+  if (!pos || !out || (n_rows > 0 && n_parts > 0 && !parts)) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  const unsigned grid = unsigned((n_slots + 255) / 256);
+  switch (out_dtype) {
+    case STM_F32: row_parts_to_slots_kernel<<<grid, 256, 0, s>>>(parts, n_parts, pos, n_slots, n_rows, static_cast<float*>(out)); break;
+    case STM_F16: row_parts_to_slots_kernel<<<grid, 256, 0, s>>>(parts, n_parts, pos, n_slots, n_rows, static_cast<f16_t*>(out)); break;
+    case STM_BF16: row_parts_to_slots_kernel<<<grid, 256, 0, s>>>(parts, n_parts, pos, n_slots, n_rows, static_cast<bf16_t*>(out)); break;
+    default: return STM_ERR_UNSUPPORTED;
   }
   return launch_status();
 }

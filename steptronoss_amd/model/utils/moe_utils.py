@@ -41,6 +41,11 @@ class Settings:
         ``validate_fused`` is set; with it the op also reproduces the reference's early-out
         for a batch in which no slot is routed (``x * token_weights.sum()``), which needs the
         routed count on the host.
+    weights_before_gemm2: ``routed_grouped_ffn`` with fp32 ``token_weights`` multiplies each
+        routed row by its weight right after the SwiGLU (in the first GEMM's epilogue) instead of
+        in the combine: the second GEMM is linear in its rows, so the sum is the same up to
+        rounding, the combine's backward shrinks to a row copy and the second GEMM's output
+        need not be kept for it.  Off: weights are applied in the combine as the reference does.
     fuse_main_grad: a weight of ``routed_grouped_ffn`` that carries an fp32 ``main_grad``
         buffer (the gradient manager's accumulator, reference
         optimizer/base_gradient_manager.py:153-155) gets its gradient added straight into that
@@ -48,6 +53,7 @@ class Settings:
         is written, re-read and added afterwards.
     """
 
+    weights_before_gemm2: bool = True
     validate: bool = True
     validate_fused: bool = False
     fuse_main_grad: bool = False
@@ -513,9 +519,9 @@ class _CombineInjective(torch.autograd.Function):
         return grad_rows, None, gw
 
 
-def _gemm_swiglu_rows(a: torch.Tensor, w1: torch.Tensor, offsets: torch.Tensor, swiglu_limit):
-    """``gate_up = a @ w1[g]^T`` and ``h = swiglu(gate_up)`` from one kernel; ``(None, None)``
-    when the fused kernel does not take the shape."""
+def _gemm_swiglu_rows(a: torch.Tensor, w1: torch.Tensor, offsets: torch.Tensor, swiglu_limit, row_scale=None):
+    """``gate_up = a @ w1[g]^T`` and ``h = swiglu(gate_up)`` (``* row_scale[r]`` when given) from
+    one kernel; ``(None, None)`` when the fused kernel does not take the shape."""
     m_cap, k = a.shape
     n_groups, two_f, _ = w1.shape
     ffn = two_f // 2
@@ -523,21 +529,24 @@ def _gemm_swiglu_rows(a: torch.Tensor, w1: torch.Tensor, offsets: torch.Tensor, 
     h = torch.empty((m_cap, ffn), device=a.device, dtype=a.dtype)
     ws = _gemm_workspace(m_cap, n_groups, a.device)
     ok = try_call(
-        "stm_grouped_gemm_swiglu", ptr(a), ptr(w1), ptr(gu), ptr(h), ptr(offsets), n_groups, m_cap, ffn, k,
+        "stm_grouped_gemm_swiglu", ptr(a), ptr(w1), ptr(gu), ptr(h), ptr(row_scale), ptr(offsets), n_groups, m_cap, ffn, k,
         int(swiglu_limit is not None), float(swiglu_limit or 0.0), dtype_code(a.dtype), ptr(ws), ws.numel(), stream(),
     )  # fmt: skip
     return (gu, h) if ok else (None, None)
 
 
-def _gemm_dswiglu_rows(gy: torch.Tensor, w2: torch.Tensor, gu: torch.Tensor, offsets: torch.Tensor, swiglu_limit):
-    """``d gate_up`` from ``d h = gy @ w2[g]`` and ``gate_up`` in one kernel (``d h`` is never
-    stored); ``None`` when the fused kernel does not take the shape."""
+def _gemm_dswiglu_rows(gy, w2, gu, offsets, swiglu_limit, row_scale=None, row_dot=None):
+    """``d gate_up`` from ``d h = gy @ w2[g]`` (``* row_scale[r]`` when given) and ``gate_up`` in
+    one kernel (``d h`` is never stored); ``row_dot`` ``[m_cap, _row_dot_parts(ffn)]`` receives
+    the partial sums of ``swiglu(gate_up)[r] . (gy @ w2[g])[r]``.  ``None`` when the fused kernel
+    does not take the shape."""
     m_cap, k = gy.shape
     n_groups, _, ffn = w2.shape
     dgu = torch.empty_like(gu)
     ws = _gemm_workspace(m_cap, n_groups, gy.device)
     ok = try_call(
-        "stm_grouped_gemm_dswiglu", ptr(gy), ptr(w2), ptr(gu), ptr(dgu), ptr(offsets), n_groups, m_cap, ffn, k,
+        "stm_grouped_gemm_dswiglu", ptr(gy), ptr(w2), ptr(gu), ptr(dgu), ptr(row_scale), ptr(row_dot), ptr(offsets),
+        n_groups, m_cap, ffn, k,
         int(swiglu_limit is not None), float(swiglu_limit or 0.0), dtype_code(gy.dtype), ptr(ws), ws.numel(), stream(),
     )  # fmt: skip
     return dgu if ok else None
@@ -558,10 +567,33 @@ def _wgrad_into_main_grad(x: torch.Tensor, y: torch.Tensor, offsets: torch.Tenso
     )  # fmt: skip
 
 
+def _row_dot_parts(ffn: int) -> int:
+    return int(_lib.load().stm_grouped_gemm_dswiglu_row_dot_parts(ffn))
+
+
+_UNIT_WEIGHTS: dict = {}
+
+
+def _unit_weights(shape, device) -> torch.Tensor:
+    key = (tuple(shape), device)
+    ones = _UNIT_WEIGHTS.get(key)
+    if ones is None:
+        _UNIT_WEIGHTS.clear()  # one shape at a time is enough
+        ones = _UNIT_WEIGHTS[key] = torch.ones(shape, device=device, dtype=torch.float32)
+    return ones
+
+
 class _FusedRoutedFFN(torch.autograd.Function):
     """route_plan -> permute -> GEMM(w1^T) -> SwiGLU -> GEMM(w2^T) -> combine in one autograd
     node: no host round trip, intermediates are sized for all ``T*K`` slots and only the rows of
-    used slots are ever touched."""
+    used slots are ever touched.
+
+    With ``settings.weights_before_gemm2`` (and fp32 weights, the fused SwiGLU kernels taking
+    the shape) row ``r = pos[t, k]`` of the SwiGLU output is multiplied by ``token_weights[t, k]``
+    before the second GEMM and the combine adds rows up unweighted.  Backward: the gradient of
+    the second GEMM's output is then a plain row copy of ``grad_out``, and
+    ``d token_weights[t, k] = grad_out[t] . y[r] = h[r] . (grad_out[t] @ w2[e])`` falls out of the
+    dgrad kernel's epilogue, which holds both factors."""
 
     @staticmethod
     def forward(ctx, w1, w2, x, token_expert_ids, token_weights, swiglu_limit, out_scale=None, out_addend=None):
@@ -581,14 +613,27 @@ class _FusedRoutedFFN(torch.autograd.Function):
             call(
                 "stm_permute_fwd", ptr(x), ptr(pos), 0, ptr(xp), T, K, H * x.element_size(), n_rows, None, stream()
             )
-            gu, h = _gemm_swiglu_rows(xp, w1, offsets, swiglu_limit)
+            w_row = None
+            if settings.weights_before_gemm2 and token_weights.dtype == torch.float32:
+                w_row = torch.empty(n_rows, device=dev, dtype=torch.float32)
+                call(
+                    "stm_slot_values_to_rows", ptr(token_weights), dtype_code(token_weights.dtype), ptr(pos), n_rows,
+                    ptr(w_row), n_rows, stream(),
+                )  # fmt: skip
+            gu, h = _gemm_swiglu_rows(xp, w1, offsets, swiglu_limit, w_row)
             if h is None:
+                w_row = None
                 gu = _gemm_rows(xp, w1, offsets, two_f, True)
                 h = swiglu_fwd_rows(gu, swiglu_limit, live)
             y = _gemm_rows(h, w2, offsets, H, True)
             addend = None if out_addend is None else out_addend.contiguous()
-            out = _combine_rows(y, pos, token_weights, out_scale, addend)
-        ctx.save_for_backward(w1, w2, xp, gu, h, y, pos, offsets, token_weights)
+            if w_row is None:
+                out = _combine_rows(y, pos, token_weights, out_scale, addend)
+                ctx.save_for_backward(w1, w2, xp, gu, h, y, pos, offsets, token_weights)
+            else:  # h and y carry the weights already
+                out = _combine_rows(y, pos, _unit_weights(pos.shape, dev), out_scale, addend)
+                ctx.save_for_backward(w1, w2, xp, gu, h, w_row, pos, offsets, token_weights)
+        ctx.weighted_rows = w_row is not None
         ctx.limit = swiglu_limit
         ctx.out_scale = out_scale
         ctx.shape = (T, H, K, E)
@@ -596,9 +641,9 @@ class _FusedRoutedFFN(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_out):
-        from steptronoss_amd.model.common.feed_forward import swiglu_bwd_rows
+        from steptronoss_amd.model.common.feed_forward import swiglu_bwd_rows, swiglu_fwd_rows
 
-        w1, w2, xp, gu, h, y, pos, offsets, token_weights = ctx.saved_tensors
+        w1, w2, xp, gu, h, y_or_w_row, pos, offsets, token_weights = ctx.saved_tensors
         T, H, K, E = ctx.shape
         dev = grad_out.device
         need_w1, need_w2, need_x, _, need_tw, _, _, need_addend = ctx.needs_input_grad
@@ -606,12 +651,41 @@ class _FusedRoutedFFN(torch.autograd.Function):
         with torch.cuda.device(dev):
             live = offsets[E:]
             go = grad_out.contiguous()
-            gy = torch.empty_like(y)
-            gtw = _combine_rows_bwd(go, y, pos, token_weights, gy, None, ctx.out_scale)
+            dgu = None
+            if ctx.weighted_rows:
+                w_row = y_or_w_row
+                n_rows = xp.shape[0]
+                if ctx.out_scale is not None:
+                    go = go * ctx.out_scale
+                gy = torch.empty_like(xp)  # rows of grad_out, one per routed slot
+                call(
+                    "stm_permute_fwd", ptr(go), ptr(pos), 0, ptr(gy), T, K, H * go.element_size(), n_rows, None, stream()
+                )
+                if need_w1 or need_x or need_tw:
+                    ffn = h.shape[1]
+                    n_parts = _row_dot_parts(ffn)
+                    parts = torch.empty((n_rows, n_parts), device=dev, dtype=torch.float32)
+                    dgu = _gemm_dswiglu_rows(gy, w2, gu, offsets, ctx.limit, w_row, parts)
+                    if dgu is None:  # the fused kernel declined: the same arithmetic, step by step
+                        dhu = _gemm_rows(gy, w2, offsets, ffn, False)
+                        parts = (swiglu_fwd_rows(gu, ctx.limit, live).float() * dhu.float()).sum(1, keepdim=True)
+                        n_parts = 1
+                        dgu = swiglu_bwd_rows(gu, (dhu.float() * w_row[:, None]).to(gu.dtype), ctx.limit, live)
+                    if need_tw:
+                        gtw = torch.empty_like(token_weights)
+                        call(
+                            "stm_row_parts_to_slots", ptr(parts), n_parts, ptr(pos), n_rows, n_rows, ptr(gtw),
+                            dtype_code(gtw.dtype), stream(),
+                        )  # fmt: skip
+            else:
+                y = y_or_w_row
+                gy = torch.empty_like(y)
+                gtw = _combine_rows_bwd(go, y, pos, token_weights, gy, None, ctx.out_scale)
             if need_w2 and not _wgrad_into_main_grad(gy, h, offsets, w2):
                 gw2 = _gemm_wgrad(gy, h, offsets, E)
             if need_w1 or need_x:
-                dgu = _gemm_dswiglu_rows(gy, w2, gu, offsets, ctx.limit)
+                if dgu is None:
+                    dgu = _gemm_dswiglu_rows(gy, w2, gu, offsets, ctx.limit)
                 if dgu is None:
                     dh = _gemm_rows(gy, w2, offsets, h.shape[1], False)
                     dgu = swiglu_bwd_rows(gu, dh, ctx.limit, live)

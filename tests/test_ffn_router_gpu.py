@@ -113,6 +113,104 @@ def test_ffn_matches_oracle(T, H, K, E, Fh, dtype, inv, tol, limit):
     _ffn_case(T, H, K, E, Fh, dtype, "own", inv, tol, limit=limit, std=0.5)
 
 
+@pytest.fixture
+def weights_before_gemm2(request):
+    old = M.settings.weights_before_gemm2
+    M.settings.weights_before_gemm2 = request.param
+    yield request.param
+    M.settings.weights_before_gemm2 = old
+
+
+@pytest.mark.parametrize("weights_before_gemm2", [True, False], indirect=True)
+@pytest.mark.parametrize(
+    "dtype,limit,inv,Fh",
+    [(torch.bfloat16, None, 0.0, 320), (torch.bfloat16, 1.0, 0.2, 320), (torch.float16, None, 0.1, 64), (torch.bfloat16, 0.8, 0.0, 768)],
+)
+def test_ffn_on_the_fused_kernels_with_weights_at_either_place(weights_before_gemm2, dtype, limit, inv, Fh):
+    # 8192 slots: the fused SwiGLU epilogues take the shape; 320 = one full column tile and a
+    # quarter of the next, so some of the row-dot parts cover dead columns only
+    from steptronoss_amd.profiling import KernelTimer
+
+    with KernelTimer() as kt:
+        _ffn_case(1024, 128, 8, 16, Fh, dtype, "own", inv, BF16_TOL, seed=3, limit=limit, std=0.3)
+    ran = set(kt.summary())
+    assert {"stm_grouped_gemm_swiglu", "stm_grouped_gemm_dswiglu"} <= ran
+    if weights_before_gemm2:
+        assert {"stm_slot_values_to_rows", "stm_row_parts_to_slots"} <= ran and "stm_unpermute_bwd_scaled" not in ran
+    else:
+        assert "stm_unpermute_bwd_scaled" in ran and "stm_slot_values_to_rows" not in ran
+
+
+@pytest.mark.parametrize("weights_before_gemm2", [True, False], indirect=True)
+def test_ffn_weight_gradient_of_slots_with_zero_weight(weights_before_gemm2):
+    # d out / d weight[t, k] = y[pos] does not vanish where the weight does
+    gen = torch.Generator().manual_seed(5)
+    T, H, K, E, Fh = 1024, 64, 4, 8, 64
+    x = (torch.randn(T, H, generator=gen) * 0.5).bfloat16()
+    w1 = (torch.randn(E, 2 * Fh, H, generator=gen) * 0.3).bfloat16()
+    w2 = (torch.randn(E, H, Fh, generator=gen) * 0.3).bfloat16()
+    ids = make_topk_ids(T, K, E, gen=gen)
+    tw = torch.rand(T, K, generator=gen)
+    tw[::3, 1] = 0.0
+    tw[5] = 0.0
+    go = torch.randn(T, H, generator=gen).bfloat16()
+    ref_in = [t.clone().float().requires_grad_(True) for t in (w1, w2, x, tw)]
+    O.routed_grouped_ffn(ref_in[0], ref_in[1], O.swiglu, ref_in[2], ids, ref_in[3]).backward(go.float())
+    got_in = [t.to(DEV).requires_grad_(True) for t in (w1, w2, x, tw)]
+    M.routed_grouped_ffn(got_in[0], got_in[1], swiglu, got_in[2], ids.to(DEV), got_in[3]).backward(go.to(DEV))
+    zero = tw == 0
+    assert float(ref_in[3].grad[zero].abs().min()) > 0
+    assert rel_l2(got_in[3].grad.cpu()[zero], ref_in[3].grad[zero]) <= BF16_TOL
+    for g, r in zip(got_in, ref_in):
+        assert rel_l2(g.grad, r.grad) <= BF16_TOL
+
+
+@pytest.mark.parametrize("weights_before_gemm2", [True, False], indirect=True)
+def test_ffn_tail_on_the_fused_kernels_matches_oracle(weights_before_gemm2):
+    gen = torch.Generator().manual_seed(6)
+    T, H, K, E, Fh = 1024, 128, 8, 16, 128
+    x = (torch.randn(T, H, generator=gen) * 0.5).bfloat16()
+    w1 = (torch.randn(E, 2 * Fh, H, generator=gen) * 0.3).bfloat16()
+    w2 = (torch.randn(E, H, Fh, generator=gen) * 0.3).bfloat16()
+    shared = torch.randn(T, H, generator=gen).bfloat16()
+    ids = make_topk_ids(T, K, E, gen=gen, invalid_frac=0.1)
+    tw = torch.rand(T, K, generator=gen)
+    go = torch.randn(T, H, generator=gen).bfloat16()
+    ref_in = [t.clone().float().requires_grad_(True) for t in (w1, w2, x, tw, shared)]
+    ref = O.routed_grouped_ffn(ref_in[0], ref_in[1], O.swiglu, ref_in[2], ids, ref_in[3]) * 2.5 + ref_in[4]
+    ref.backward(go.float())
+    got_in = [t.to(DEV).requires_grad_(True) for t in (w1, w2, x, tw, shared)]
+    out = M.hip_routed_grouped_ffn(
+        got_in[0], got_in[1], swiglu, got_in[2], ids.to(DEV), got_in[3], out_scale=2.5, out_addend=got_in[4]
+    )
+    out.backward(go.to(DEV))
+    assert rel_l2(out, ref) <= BF16_TOL
+    for g, r in zip(got_in, ref_in):
+        assert rel_l2(g.grad, r.grad) <= BF16_TOL
+
+
+def test_slot_and_row_order_helpers():
+    gen = torch.Generator().manual_seed(7)
+    T, K, E = 300, 4, 8
+    ids = make_topk_ids(T, K, E, gen=gen, invalid_frac=0.2).to(DEV)
+    pos = M.index_compute(ids, M.histogram(ids, E))
+    n_rows = T * K
+    for dt in (torch.float32, torch.bfloat16, torch.float16):
+        vals = torch.rand(T, K, generator=gen).to(dt).to(DEV)
+        rows = torch.full((n_rows,), -1.0, device=DEV)
+        M.call("stm_slot_values_to_rows", M.ptr(vals), M.dtype_code(dt), M.ptr(pos), n_rows, M.ptr(rows), n_rows, M.stream())
+        expect = torch.full((n_rows,), -1.0, device=DEV)
+        valid = pos >= 0
+        expect[pos[valid].long()] = vals[valid].float()
+        assert torch.equal(rows, expect)
+        parts = torch.randn(n_rows, 3, generator=gen).to(DEV)
+        out = torch.empty(T, K, device=DEV, dtype=dt)
+        M.call("stm_row_parts_to_slots", M.ptr(parts), 3, M.ptr(pos), n_rows, n_rows, M.ptr(out), M.dtype_code(dt), M.stream())
+        want = torch.zeros(T, K, device=DEV)
+        want[valid] = ((parts[:, 0] + parts[:, 1]) + parts[:, 2])[pos[valid].long()]
+        assert torch.equal(out, want.to(dt))
+
+
 def test_ffn_experts_without_tokens():
     # only experts 0 and 5 are used: the other weight gradients must be exactly zero
     gen = torch.Generator().manual_seed(1)
