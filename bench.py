@@ -39,7 +39,7 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 # from hardware counters collected in separate profiler runs of this script (FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB copies of
 # --traffic-probe); the summaries of those runs are kept under profiles/.  None = not measured.
-MEASURED_GEMM_TRAFFIC_BYTES = {"c2": 2.455e9, "c3": None, "c4": None}
+MEASURED_GEMM_TRAFFIC_BYTES = {"c2": 2.465e9, "c3": None, "c4": None}
 
 WORKLOADS = {
     "c1": dict(T=4096, H=1024, E=8, K=2, F=2048, sigmoid=False, norm=False, n_group=1, topk_group=1, std=0.02, dtype="fp32"),
@@ -198,6 +198,26 @@ def main():
         "avg_launch_us": avg_launch_ms * 1e3,
         "launches_per_step": gemm_calls / args.steps,
     }
+
+    # The stand-alone combine op (moe_weighted_gather, weights applied in the combine), outside
+    # the timed steps: the fused FFN's backward replaces its backward kernel by a row copy.
+    from steptronoss_amd.model.utils.moe_utils import histogram, index_compute, moe_weighted_gather
+
+    with torch.no_grad():
+        ids, weights, _aux, _hist = forward_router(
+            logits, K, use_sigmoid=cfg["sigmoid"], norm_expert_weight=cfg["norm"], n_group=cfg["n_group"],
+            topk_group=cfg["topk_group"],
+        )  # fmt: skip
+    pos = index_compute(ids, histogram(ids, E))
+    rows = torch.randn(N, H, device=dev, dtype=x.dtype).requires_grad_(True)
+    slot_weights = weights.detach().clone().requires_grad_(True)
+    with KernelTimer() as kt_op:
+        for _ in range(5):
+            rows.grad = slot_weights.grad = None
+            moe_weighted_gather(rows, pos, slot_weights).backward(go)
+    for name, t in kt_op.summary().items():
+        timing.setdefault(name, t)
+    del rows, slot_weights
 
     def bw(names, nbytes):
         t = next((timing[n] for n in names.split("|") if n in timing and timing[n]["calls"]), None)
