@@ -1,0 +1,162 @@
+"""Randomised differential test: every op of the backend against the CPU oracle on shapes drawn at
+random, including the awkward ones (no tokens, one expert, one column, odd widths, every slot
+unused, int32 ids, batch sizes on the host or the device).  The "large" draws reach the MFMA
+kernels and the fused SwiGLU epilogues.  Tolerances: ids / positions / copies bit-exact; fp32
+1e-4; 16-bit storage 1.5e-2 (rel. L2), twice that for quantities that sum many rounded products.
+"""
+
+import functools
+import random
+
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from steptronoss_amd.model.common.feed_forward import swiglu
+from steptronoss_amd.model.common.moe_block import forward_router
+from steptronoss_amd.model.utils import moe_utils as M
+from steptronoss_amd.utils.optimizable import set_optimization
+from tests.helpers import make_topk_ids, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(autouse=True)
+def _select_backend():
+    set_optimization("hip_gfx950")
+    yield
+    set_optimization()
+
+
+def _tol(dt):
+    return 1e-4 if dt == torch.float32 else 1.5e-2
+
+
+def _draw(rng, large):
+    if large:
+        c = dict(
+            T=rng.choice([1024, 1500, 2048, 4100]), K=rng.choice([4, 8]), E=rng.choice([4, 8, 16, 33]),
+            H=rng.choice([64, 96, 128, 256]), F=rng.choice([64, 72, 128, 320]),
+            dt=rng.choice([torch.bfloat16, torch.float16]), inv=rng.choice([0.0, 0.1]),
+        )  # fmt: skip
+    else:
+        c = dict(
+            T=rng.choice([0, 1, 2, 3, 7, 33, 64, 100, 257, 600, 1100]), K=rng.choice([1, 1, 2, 3, 4, 8]),
+            E=rng.choice([1, 2, 3, 5, 8, 16, 37, 64]), H=rng.choice([1, 2, 8, 24, 56, 64, 100, 128, 136]),
+            F=rng.choice([4, 8, 24, 32, 64, 72]), dt=rng.choice([torch.float32, torch.bfloat16, torch.float16]),
+            inv=rng.choice([0.0, 0.0, 0.2, 1.0]),
+        )  # fmt: skip
+    c["K"] = min(c["K"], c["E"])
+    c["idt"] = rng.choice([torch.int32, torch.int64])
+    return c
+
+
+def _run_case(rng, c, seed):
+    T, K, E, H, Fh, dt = c["T"], c["K"], c["E"], c["H"], c["F"], c["dt"]
+    gen = torch.Generator().manual_seed(seed)
+    ids = make_topk_ids(T, K, E, gen=gen, invalid_frac=c["inv"], dtype=c["idt"])
+    n_rows = int((ids >= 0).sum())
+
+    # ---- histogram, index_compute: bit-exact
+    h_ref = O.histogram(ids, E)
+    h = M.histogram(ids.to(DEV), E)
+    assert torch.equal(h.cpu(), h_ref)
+    p_ref = O.index_compute(ids, h_ref)
+    p = M.index_compute(ids.to(DEV), h)
+    assert torch.equal(p.cpu(), p_ref)
+
+    # ---- moe_scatter: rows are copies; backward sums K rows
+    x = torch.randn(T, H, generator=gen).to(dt)
+    xr, xg = x.clone().float().requires_grad_(True), x.to(DEV).requires_grad_(True)
+    s_ref, s = O.moe_scatter(xr, p_ref), M.moe_scatter(xg, p)
+    assert s.shape == s_ref.shape and torch.equal(s.float().cpu(), s_ref.to(dt).float())
+    go = torch.randn(s_ref.shape, generator=gen).to(dt)
+    s_ref.backward(go.float())
+    s.backward(go.to(DEV))
+    if T > 0:
+        assert rel_l2(xg.grad, xr.grad) <= _tol(dt)
+
+    # ---- moe_weighted_gather (the reference raises on an empty input with slots to fill)
+    rows = torch.randn(s_ref.shape[0], H, generator=gen).to(dt)
+    w = torch.rand(T, K, generator=gen)
+    go_t = torch.randn(T, H, generator=gen).to(dt)
+    if s_ref.shape[0] > 0 or T * K == 0:
+        rr, wr = rows.clone().float().requires_grad_(True), w.clone().requires_grad_(True)
+        rg, wg = rows.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+        g_ref, g = O.moe_weighted_gather(rr, p_ref, wr), M.moe_weighted_gather(rg, p, wg)
+        assert g.shape == g_ref.shape and (T == 0 or rel_l2(g, g_ref) <= _tol(dt))
+        g_ref.backward(go_t.float())
+        g.backward(go_t.to(DEV))
+        if n_rows > 0:
+            assert rel_l2(rg.grad, rr.grad) <= _tol(dt)
+            assert rel_l2(wg.grad, wr.grad) <= 2 * _tol(dt)
+
+    # ---- grouped_gemm, both weight layouts, batch sizes on either side
+    sizes = h_ref.to(torch.int64)
+    for trans_b in (True, False):
+        a = (torch.randn(n_rows, H, generator=gen) * 0.5).to(dt)
+        b = (torch.randn(*((E, Fh, H) if trans_b else (E, H, Fh)), generator=gen) * 0.5).to(dt)
+        ar, br = a.clone().float().requires_grad_(True), b.clone().float().requires_grad_(True)
+        ag, bg = a.to(DEV).requires_grad_(True), b.to(DEV).requires_grad_(True)
+        c_ref = O.grouped_gemm(ar, br, sizes, trans_b)
+        out = M.grouped_gemm(ag, bg, sizes.to(DEV) if rng.random() < 0.5 else sizes, trans_b)
+        assert out.shape == c_ref.shape and (n_rows == 0 or rel_l2(out, c_ref) <= _tol(dt))
+        gc = torch.randn(c_ref.shape, generator=gen).to(dt)
+        c_ref.backward(gc.float())
+        out.backward(gc.to(DEV))
+        if n_rows > 0:
+            assert rel_l2(ag.grad, ar.grad) <= _tol(dt)
+        assert rel_l2(bg.grad, br.grad) <= _tol(dt)
+
+    # ---- routed_grouped_ffn
+    if T > 0:
+        w1 = (torch.randn(E, 2 * Fh, H, generator=gen) * 0.3).to(dt)
+        w2 = (torch.randn(E, H, Fh, generator=gen) * 0.3).to(dt)
+        limit = rng.choice([None, None, 1.0])
+
+        def ref_act(hh):  # the clamp decides on the stored (rounded) value, as the kernels do
+            if limit is not None and dt != torch.float32:
+                hh = hh + (hh.to(dt).float() - hh).detach()
+            return O.swiglu(hh, limit)
+
+        ref_in = [t.clone().float().requires_grad_(True) for t in (w1, w2, x, w)]
+        O.routed_grouped_ffn(ref_in[0], ref_in[1], ref_act, ref_in[2], ids, ref_in[3]).backward(go_t.float())
+        got_in = [t.to(DEV).requires_grad_(True) for t in (w1, w2, x, w)]
+        act = functools.partial(swiglu, swiglu_limit=limit)
+        M.routed_grouped_ffn(got_in[0], got_in[1], act, got_in[2], ids.to(DEV), got_in[3]).backward(go_t.to(DEV))
+        if n_rows > 0:
+            for gt, rf in zip(got_in, ref_in):
+                assert rel_l2(gt.grad, rf.grad) <= 2 * _tol(dt)
+
+    # ---- router on fp32 logits
+    if T > 0 and E >= 2:
+        sig = rng.random() < 0.5
+        ng, tg = (4, rng.choice([1, 2, 3])) if E % 4 == 0 and rng.random() < 0.5 else (1, 1)
+        k_r = min(K, E if ng == 1 else (E // ng) * tg)
+        logits = torch.randn(T, E, generator=gen)
+        bias = torch.randn(E, generator=gen) * 0.1 if rng.random() < 0.3 else None
+        lr, lg = logits.clone().requires_grad_(True), logits.to(DEV).requires_grad_(True)
+        kw = dict(use_sigmoid=sig, norm_expert_weight=True, n_group=ng, topk_group=tg)
+        r_ids, r_w, r_aux = O.forward_router(lr, k_r, balance_bias=bias, **kw)[:3]
+        g_ids, g_w, g_aux, _ = forward_router(lg, k_r, balance_bias=None if bias is None else bias.to(DEV), **kw)
+        if not torch.equal(g_ids.cpu(), r_ids):  # scores one ulp apart may swap two neighbours
+            assert float((g_ids.cpu() != r_ids).float().mean()) < 0.002
+            return
+        assert torch.allclose(g_w.detach().cpu(), r_w.detach(), atol=2e-6, rtol=1e-5)
+        assert abs(float(g_aux.detach()) - float(r_aux.detach())) <= 1e-4 * max(1.0, abs(float(r_aux.detach())))
+        gw = torch.randn(T, k_r, generator=gen)
+        torch.autograd.backward([r_w, r_aux], [gw, torch.tensor(0.5)])
+        torch.autograd.backward([g_w, g_aux], [gw.to(DEV), torch.tensor(0.5, device=DEV)])
+        assert rel_l2(lg.grad, lr.grad) <= 1e-4
+
+
+@pytest.mark.parametrize("seed,large,count", [(0, False, 60), (1, False, 60), (2, True, 10)])
+def test_random_shapes_match_the_oracle(seed, large, count):
+    rng = random.Random(seed)
+    for it in range(count):
+        case = _draw(rng, large)
+        try:
+            _run_case(rng, case, 1000 * seed + it)
+        except AssertionError as err:
+            raise AssertionError(f"case {it} of seed {seed}: {case}") from err
