@@ -204,7 +204,9 @@ int stm_grouped_gemm(const void* a, const void* b, void* c, const int32_t* offse
  *                             and h [m_cap, ffn] = swiglu(gate_up), both stored;
  *   stm_grouped_gemm_dswiglu: d gate_up [m_cap, 2*ffn] from d h = grad_y [m_cap, k] * w2[g]
  *                             (w2 [G, k, ffn]) and gate_up; d h itself is never stored.
- * Results are bit-identical to stm_grouped_gemm followed by stm_swiglu_fwd / stm_swiglu_bwd.
+ * Results are those of stm_grouped_gemm followed by stm_swiglu_fwd / stm_swiglu_bwd (the same
+ * per-element code: bit-identical in bf16; in fp16 single results may differ by one step where the
+ * compiler merges a last multiplication with the conversion in one kernel and not in the other).
  * Return STM_ERR_UNSUPPORTED for shapes the fused kernels do not take (k not a multiple of 32,
  * ffn not a multiple of 8, fewer than 4096 rows, fp32): callers then use the unfused pair.
  * Workspace as for stm_grouped_gemm.

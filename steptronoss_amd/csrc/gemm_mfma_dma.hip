@@ -668,11 +668,17 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
             stage([&](int jj, int q, int e) { return acc[i][2 + jj][q * 4 + e]; });
             store_round(rsrc_c, row_bytes_c, up_bytes);
             const float scale = row_scale_of(row0 + r);  // in the accumulators a lane owns one row
-            stage([&](int jj, int q, int e) {  // from the values as stored: h = swiglu(rounded gate, rounded up)
-              return swiglu_value(round_to<T>(acc[i][jj][q * 4 + e]), round_to<T>(acc[i][2 + jj][q * 4 + e]), has_limit,
-                                  limit) *
-                     scale;
-            });
+            auto stage_h = [&](auto limit_tag) {  // from the values as stored: h = swiglu(rounded gate, rounded up)
+              stage([&](int jj, int q, int e) {
+                return swiglu_value_t<decltype(limit_tag)::value>(round_to<T>(acc[i][jj][q * 4 + e]),
+                                                                  round_to<T>(acc[i][2 + jj][q * 4 + e]), limit) *
+                       scale;
+              });
+            };
+            if (has_limit)
+              stage_h(std::true_type{});
+            else
+              stage_h(std::false_type{});
             store_round(rsrc_2, row_bytes_2, 0u);
           }
         } else {
@@ -712,16 +718,24 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
                 const uint4 d = staged(it);
                 Pack8<T> dv = __builtin_bit_cast(Pack8<T>, d), gv = __builtin_bit_cast(Pack8<T>, gate[it]),
                          uv = __builtin_bit_cast(Pack8<T>, up[it]), og, ou;
+                // (one uniform branch per eight elements: the clamps are compiled away when there is
+                // no limit; a branch around all four `it` would let the four be interleaved and
+                // spill registers)
+                auto eight = [&](auto limit_tag) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                  float dg, du;
-                  const float g = to_float(gv.v[e]), u = to_float(uv.v[e]), d = to_float(dv.v[e]);
-                  float h_val;
-                  swiglu_grads(g, u, d * scale[it], has_limit, limit, dg, du, h_val);
-                  dot[it] += h_val * d;
-                  og.v[e] = from_float<T>(dg);
-                  ou.v[e] = from_float<T>(du);
-                }
+                  for (int e = 0; e < 8; ++e) {
+                    float dg, du, h_val;
+                    const float g = to_float(gv.v[e]), u = to_float(uv.v[e]), dh = to_float(dv.v[e]);
+                    swiglu_grads_t<decltype(limit_tag)::value>(g, u, dh * scale[it], limit, dg, du, h_val);
+                    dot[it] += h_val * dh;
+                    og.v[e] = from_float<T>(dg);
+                    ou.v[e] = from_float<T>(du);
+                  }
+                };
+                if (has_limit)
+                  eight(std::true_type{});
+                else
+                  eight(std::false_type{});
                 const uint32_t at =
                     col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset;
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, og), rsrc_c, at, 0, 0);

@@ -11,10 +11,11 @@ struct alignas(sizeof(T) * VEC) Pack {
   T v[VEC];
 };
 
-template <typename T, int VEC>
+// LIMIT is a template argument so that the code without a limit carries no clamps; the GEMM
+// epilogues instantiate the same per-element functions.
+template <typename T, int VEC, bool LIMIT>
 __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const T* __restrict__ gu, T* __restrict__ h, int64_t rows,
-                                                         int64_t f, const int32_t* __restrict__ rows_dev,
-                                                         bool has_limit, float limit) {
+                                                         int64_t f, const int32_t* __restrict__ rows_dev, float limit) {
   using P = Pack<T, VEC>;
   const int64_t per_row = f / VEC;
   const int64_t live = rows_dev ? (rows_dev[0] < rows ? rows_dev[0] : rows) : rows;
@@ -26,17 +27,16 @@ __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const T* __restrict__ g
     P o;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      o.v[j] = from_float<T>(swiglu_value(to_float(g.v[j]), to_float(u.v[j]), has_limit, limit));
+      o.v[j] = from_float<T>(swiglu_value_t<LIMIT>(to_float(g.v[j]), to_float(u.v[j]), limit));
     }
     *reinterpret_cast<P*>(h + r * f + c) = o;
   }
 }
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool LIMIT>
 __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ gu, const T* __restrict__ dh,
                                                          T* __restrict__ dgu, int64_t rows, int64_t f,
-                                                         const int32_t* __restrict__ rows_dev, bool has_limit,
-                                                         float limit) {
+                                                         const int32_t* __restrict__ rows_dev, float limit) {
   using P = Pack<T, VEC>;
   const int64_t per_row = f / VEC;
   const int64_t live = rows_dev ? (rows_dev[0] < rows ? rows_dev[0] : rows) : rows;
@@ -49,8 +49,8 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ g
     P og, ou;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      float dg, du;
-      swiglu_grads(to_float(g.v[j]), to_float(u.v[j]), to_float(d.v[j]), has_limit, limit, dg, du);
+      float dg, du, value;
+      swiglu_grads_t<LIMIT>(to_float(g.v[j]), to_float(u.v[j]), to_float(d.v[j]), limit, dg, du, value);
       og.v[j] = from_float<T>(dg);
       ou.v[j] = from_float<T>(du);
     }
@@ -64,34 +64,45 @@ inline unsigned grid_for(int64_t work_items) {
   return unsigned(blocks < 1 ? 1 : (blocks > 65536 ? 65536 : blocks));
 }
 
-template <typename T>
-int fwd_typed(const void* gu, void* h, int64_t rows, int64_t f, const int32_t* rows_dev, int has_limit, float limit,
-              hipStream_t s) {
+template <typename T, bool LIMIT>
+int fwd_limit(const void* gu, void* h, int64_t rows, int64_t f, const int32_t* rows_dev, float limit, hipStream_t s) {
   constexpr int W = 16 / int(sizeof(T));
   const bool vec = f % W == 0 && aligned_to(gu, 16) && aligned_to(h, 16);
   if (vec)
-    swiglu_fwd_kernel<T, W><<<grid_for(rows * (f / W)), 256, 0, s>>>(static_cast<const T*>(gu), static_cast<T*>(h),
-                                                                     rows, f, rows_dev, has_limit != 0, limit);
+    swiglu_fwd_kernel<T, W, LIMIT><<<grid_for(rows * (f / W)), 256, 0, s>>>(static_cast<const T*>(gu),
+                                                                            static_cast<T*>(h), rows, f, rows_dev, limit);
   else
-    swiglu_fwd_kernel<T, 1><<<grid_for(rows * f), 256, 0, s>>>(static_cast<const T*>(gu), static_cast<T*>(h), rows, f,
-                                                               rows_dev, has_limit != 0, limit);
+    swiglu_fwd_kernel<T, 1, LIMIT><<<grid_for(rows * f), 256, 0, s>>>(static_cast<const T*>(gu), static_cast<T*>(h),
+                                                                      rows, f, rows_dev, limit);
+  return launch_status();
+}
+
+template <typename T>
+int fwd_typed(const void* gu, void* h, int64_t rows, int64_t f, const int32_t* rows_dev, int has_limit, float limit,
+              hipStream_t s) {
+  return has_limit ? fwd_limit<T, true>(gu, h, rows, f, rows_dev, limit, s)
+                   : fwd_limit<T, false>(gu, h, rows, f, rows_dev, limit, s);
+}
+
+template <typename T, bool LIMIT>
+int bwd_limit(const void* gu, const void* dh, void* dgu, int64_t rows, int64_t f, const int32_t* rows_dev, float limit,
+              hipStream_t s) {
+  constexpr int W = 16 / int(sizeof(T));
+  const bool vec = f % W == 0 && aligned_to(gu, 16) && aligned_to(dh, 16) && aligned_to(dgu, 16);
+  if (vec)
+    swiglu_bwd_kernel<T, W, LIMIT><<<grid_for(rows * (f / W)), 256, 0, s>>>(
+        static_cast<const T*>(gu), static_cast<const T*>(dh), static_cast<T*>(dgu), rows, f, rows_dev, limit);
+  else
+    swiglu_bwd_kernel<T, 1, LIMIT><<<grid_for(rows * f), 256, 0, s>>>(
+        static_cast<const T*>(gu), static_cast<const T*>(dh), static_cast<T*>(dgu), rows, f, rows_dev, limit);
   return launch_status();
 }
 
 template <typename T>
 int bwd_typed(const void* gu, const void* dh, void* dgu, int64_t rows, int64_t f, const int32_t* rows_dev,
               int has_limit, float limit, hipStream_t s) {
-  constexpr int W = 16 / int(sizeof(T));
-  const bool vec = f % W == 0 && aligned_to(gu, 16) && aligned_to(dh, 16) && aligned_to(dgu, 16);
-  if (vec)
-    swiglu_bwd_kernel<T, W><<<grid_for(rows * (f / W)), 256, 0, s>>>(
-        static_cast<const T*>(gu), static_cast<const T*>(dh), static_cast<T*>(dgu), rows, f, rows_dev, has_limit != 0,
-        limit);
-  else
-    swiglu_bwd_kernel<T, 1><<<grid_for(rows * f), 256, 0, s>>>(static_cast<const T*>(gu), static_cast<const T*>(dh),
-                                                               static_cast<T*>(dgu), rows, f, rows_dev, has_limit != 0,
-                                                               limit);
-  return launch_status();
+  return has_limit ? bwd_limit<T, true>(gu, dh, dgu, rows, f, rows_dev, limit, s)
+                   : bwd_limit<T, false>(gu, dh, dgu, rows, f, rows_dev, limit, s);
 }
 
 }  // namespace

@@ -120,17 +120,26 @@ def test_fused_swiglu_epilogues_match_the_unfused_pair(sizes, k, ffn, dtype, lim
     w2 = (torch.randn(E, k, ffn, generator=gen) * 0.2).to(dtype).to(DEV)
     gy = torch.randn(m, k, generator=gen).to(dtype).to(DEV)
     offsets = M._group_offsets(torch.tensor(sizes), torch.device(DEV))
+    def same(got, ref):
+        # bf16: the same bits.  fp16: the compiler may merge a result's last multiplication with
+        # its conversion to fp16 (one rounding, v_fma_mixlo_f16) in one kernel and not in the
+        # other (two roundings), so single results may sit one fp16 step apart.
+        if dtype == torch.bfloat16:
+            return torch.equal(got, ref)
+        g, r = got.float(), ref.float()
+        return bool(((g - r).abs() <= 2.0**-10 * torch.maximum(g.abs(), r.abs()) + 1e-7).all())
+
     gu, h = M._gemm_swiglu_rows(a, w1, offsets, limit)
     assert h is not None, "the fused kernel declined a shape it should take"
     gu_ref = M._gemm_rows(a, w1, offsets, 2 * ffn, True)
     h_ref = swiglu_fwd_rows(gu_ref, limit)
     assert torch.equal(gu, gu_ref)
-    assert torch.equal(h, h_ref)
+    assert same(h, h_ref)
     dgu = M._gemm_dswiglu_rows(gy, w2, gu_ref, offsets, limit)
     assert dgu is not None
     dh_ref = M._gemm_rows(gy, w2, offsets, ffn, False)
     dgu_ref = swiglu_bwd_rows(gu_ref, dh_ref, limit)
-    assert torch.equal(dgu, dgu_ref)
+    assert same(dgu, dgu_ref)
     # and against the oracle in fp32
     ref32 = O.swiglu(O.grouped_gemm(a.cpu().float(), w1.cpu().float(), torch.tensor(sizes), trans_b=True), limit)
     assert rel_l2(h, ref32) <= 1e-2
