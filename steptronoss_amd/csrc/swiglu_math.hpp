@@ -7,7 +7,10 @@
 
 namespace stm {
 
-__device__ __forceinline__ float swiglu_sigmoid(float x) { return 1.f / (1.f + __expf(-x)); }
+// 1 / (1 + e^-x) with the hardware exponential and reciprocal (each within one fp32 ulp; an
+// IEEE-rounded division would cost ten instructions per element of an epilogue that is bound by
+// instruction issue, for a digit that the 16-bit rounding of the result discards).
+__device__ __forceinline__ float swiglu_sigmoid(float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
 
 // kLimit = false compiles the clamps away; callers branch once (or are instantiated) per case
 // instead of once per element.
