@@ -39,7 +39,7 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 # from hardware counters collected in separate profiler runs of this script (FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB copies of
 # --traffic-probe); the summaries of those runs are kept under profiles/.  None = not measured.
-MEASURED_GEMM_TRAFFIC_BYTES = {"c2": 2.465e9, "c3": None, "c4": None}
+MEASURED_GEMM_TRAFFIC_BYTES = {"c2": 2.48e9, "c3": None, "c4": None}
 
 WORKLOADS = {
     "c1": dict(T=4096, H=1024, E=8, K=2, F=2048, sigmoid=False, norm=False, n_group=1, topk_group=1, std=0.02, dtype="fp32"),
