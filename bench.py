@@ -49,6 +49,16 @@ WORKLOADS = {
 }
 
 
+def zipf_logit_bias(E, s, gen):
+    """``log`` of a Zipf(s) popularity profile laid over a seeded permutation of the experts;
+    added to every token's logits it skews the routing (workload c3)."""
+    pop = torch.arange(1, E + 1, dtype=torch.float64) ** (-s)
+    pop = pop / pop.sum()
+    bias = torch.empty(E, dtype=torch.float64)
+    bias[torch.randperm(E, generator=gen)] = torch.log(pop)
+    return bias.float()
+
+
 def make_inputs(cfg, seed, device):
     gen = torch.Generator(device=device).manual_seed(seed)
     T, H, E, F = cfg["T"], cfg["H"], cfg["E"], cfg["F"]
@@ -61,8 +71,6 @@ def make_inputs(cfg, seed, device):
         w2[e] = (torch.randn(H, F, generator=gen, device=device) * cfg["std"]).to(bf)
     logits = torch.randn(T, E, generator=gen, device=device)
     if "zipf" in cfg:
-        from oracle.moe_oracle import zipf_logit_bias
-
         logits = logits + zipf_logit_bias(E, cfg["zipf"], torch.Generator().manual_seed(seed)).to(device)
     go = torch.randn(T, H, generator=gen, device=device).to(bf)
     return x, w1, w2, logits, go
