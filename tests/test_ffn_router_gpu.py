@@ -189,6 +189,32 @@ def test_ffn_tail_on_the_fused_kernels_matches_oracle(weights_before_gemm2):
         assert rel_l2(g.grad, r.grad) <= BF16_TOL
 
 
+def test_ffn_backward_when_the_fused_dgrad_declines(monkeypatch):
+    # the forward put the weights on the rows; should the fused dgrad kernel ever decline, the
+    # backward does the same arithmetic step by step
+    gen = torch.Generator().manual_seed(11)
+    T, H, K, E, Fh = 1024, 64, 4, 8, 64
+    x = (torch.randn(T, H, generator=gen) * 0.5).bfloat16()
+    w1 = (torch.randn(E, 2 * Fh, H, generator=gen) * 0.3).bfloat16()
+    w2 = (torch.randn(E, H, Fh, generator=gen) * 0.3).bfloat16()
+    ids = make_topk_ids(T, K, E, gen=gen, invalid_frac=0.1).to(DEV)
+    tw = torch.rand(T, K, generator=gen)
+    go = torch.randn(T, H, generator=gen).bfloat16().to(DEV)
+
+    def run():
+        ins = [t.to(DEV).requires_grad_(True) for t in (w1, w2, x, tw)]
+        M.routed_grouped_ffn(ins[0], ins[1], swiglu, ins[2], ids, ins[3]).backward(go)
+        return [t.grad for t in ins]
+
+    fused = run()
+    real = M._gemm_dswiglu_rows
+    monkeypatch.setattr(M, "_gemm_dswiglu_rows", lambda *a, **k: None)
+    stepwise = run()
+    monkeypatch.setattr(M, "_gemm_dswiglu_rows", real)
+    for a, b in zip(fused, stepwise):
+        assert rel_l2(a, b.float()) <= 5e-3
+
+
 def test_slot_and_row_order_helpers():
     gen = torch.Generator().manual_seed(7)
     T, K, E = 300, 4, 8
