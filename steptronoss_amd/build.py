@@ -83,5 +83,25 @@ def build_library(verbose: bool = True, jobs: int = 8) -> Path:
     return LIB_PATH
 
 
+def build_host_check(verbose: bool = True) -> Path:
+    """Compile ``tests/capi_host/host_check.cpp`` (a torch-free host of the C ABI, used by the GPU
+    tests) into a small shared library next to its source, linked against the main library."""
+    src = PKG.parent / "tests" / "capi_host" / "host_check.cpp"
+    out = src.with_name("libstm_host_check.so")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [  # host code only: the plain C++ compiler, the HIP runtime API headers and library
+        "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__", f"-I{rocm}/include", str(src),
+        "-o", str(out), f"-L{LIB_DIR}", "-lsteptron_moe_gfx950", "-Wl,-rpath,$ORIGIN/../../steptronoss_amd/lib",
+        f"-L{rocm}/lib", "-lamdhip64", f"-Wl,-rpath,{rocm}/lib",
+    ]  # fmt: skip
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("host check build failed:\n" + proc.stdout + proc.stderr)
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 if __name__ == "__main__":
     build_library()
+    build_host_check()
