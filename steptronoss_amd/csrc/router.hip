@@ -14,7 +14,7 @@ namespace stm {
 namespace {
 
 constexpr int kMaxPerLane = 16;  // experts per lane  => E <= 1024
-constexpr int kRouterWaves = 4;
+constexpr int kRouterWaves = 16;  // 1024 threads: fewer, larger workgroups = fewer partial rows for the finish kernel
 constexpr int kMaxGroupsRouted = 64;
 constexpr int kMaxTopK = 64;
 
@@ -396,7 +396,7 @@ __global__ __launch_bounds__(1024) void router_bias_update_kernel(int32_t* __res
 
 inline int router_blocks(int64_t n_tokens) {
   const int64_t want = (n_tokens + kRouterWaves - 1) / kRouterWaves;
-  return int(want < 1 ? 1 : (want > 1024 ? 1024 : want));
+  return int(want < 1 ? 1 : (want > 512 ? 512 : want));
 }
 
 inline int check_router_args(const RouterArgs& a) {
