@@ -105,7 +105,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_fwd_kernel(RouterA
     // ---- group-limited routing: keep the topk_group groups with the largest top-2 sums
     if (a.n_group > 1) {
       uint64_t keep = 0;
-      float gscore[kMaxGroupsRouted];
+      float my_gscore = -INFINITY;  // lane g keeps the score of group g (n_group <= 64)
       for (int g = 0; g < a.n_group; ++g) {
         float best = -INFINITY;
 #pragma unroll
@@ -128,19 +128,15 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_fwd_kernel(RouterA
         }
         n_top = wave_sum(n_top);
         second = wave_max(second);
-        gscore[g] = per_group >= 2 ? top1 + (n_top >= 2 ? top1 : second) : top1;
+        const float gscore = per_group >= 2 ? top1 + (n_top >= 2 ? top1 : second) : top1;
+        if (lane == g) my_gscore = gscore;
       }
-      for (int r = 0; r < a.topk_group; ++r) {
-        int pick = -1;
-        float best = 0.f;
-        for (int g = 0; g < a.n_group; ++g) {
-          if ((keep >> g) & 1) continue;
-          if (pick < 0 || gscore[g] > best) {
-            pick = g;
-            best = gscore[g];
-          }
-        }
-        if (pick >= 0) keep |= 1ull << pick;
+      for (int r = 0; r < a.topk_group; ++r) {  // largest score first, equal scores: lower group
+        const bool free_group = lane < a.n_group && !((keep >> lane) & 1);
+        float best = free_group ? my_gscore : -INFINITY;
+        int pick = free_group ? lane : INT32_MAX;
+        wave_argmax(best, pick);
+        if (pick != INT32_MAX) keep |= 1ull << pick;
       }
 #pragma unroll
       for (int j = 0; j < V; ++j) {
