@@ -24,6 +24,39 @@ def test_header_symbols_are_exported_and_bound():
     assert sorted(_lib.SIGNATURES) == names, "ctypes table and header disagree"
 
 
+def _declared_prototypes():
+    """name -> (return kind, [parameter kinds]) from the header; kinds: 'ptr', 'int', 'i64', 'size', 'float'."""
+    text = (ROOT / "include" / "steptron_moe.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+
+    def kind(decl):
+        decl = decl.strip()
+        if "*" in decl or decl.startswith("stm_stream_t"):
+            return "ptr"
+        base = decl.rsplit(" ", 1)[0] if " " in decl else decl
+        return {"int": "int", "int64_t": "i64", "size_t": "size", "float": "float"}[base.replace("const ", "").strip()]
+
+    out = {}
+    for ret, name, params in re.findall(r"\b([a-z_0-9]+\s*\*?)\s+(stm_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text):
+        params = params.strip()
+        plist = [] if params in ("", "void") else [kind(x) for x in params.split(",")]
+        out[name] = ("ptr" if "*" in ret else kind(ret.strip() + " x"), plist)
+    return out
+
+
+def test_ctypes_table_matches_the_header_prototypes():
+    kinds = {
+        ctypes.c_void_p: "ptr", ctypes.c_char_p: "ptr", ctypes.c_int: "int", ctypes.c_int64: "i64",
+        ctypes.c_size_t: "size", ctypes.c_float: "float",
+    }  # fmt: skip
+    protos = _declared_prototypes()
+    assert sorted(protos) == sorted(_lib.SIGNATURES)
+    for name, (res, args) in _lib.SIGNATURES.items():
+        want_res, want_args = protos[name]
+        assert kinds[res] == want_res, f"{name}: return type"
+        assert [kinds[a] for a in args] == want_args, f"{name}: {[kinds[a] for a in args]} vs header {want_args}"
+
+
 def test_version_and_status_strings():
     lib = _lib.load()
     assert lib.stm_abi_version() >= 1
