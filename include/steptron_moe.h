@@ -280,6 +280,19 @@ int stm_swiglu_bwd(const void* gate_up, const void* grad_out, void* grad_gate_up
  *   k must be a multiple of 128.  Workspace as for stm_grouped_gemm. */
 int stm_quantize_e4m3_1x128(const void* x, int dtype, int64_t rows, int64_t cols, uint8_t* codes_out, float* scales_out,
                             stm_stream_t stream);
+
+/* The same with power-of-two scales (the smallest power of two >= amax/448), which the block-scaled
+ * matrix instruction of gfx950 applies in hardware, stored block-major:
+ * scales_by_block[kb * rows + r].  stm_grouped_gemm_fp8_pow2 is the grouped GEMM on such operands
+ * (a_scales_by_block [k/128, m_cap], b_scales_by_block [k/128, G*n]; c in bf16 or fp16) on the
+ * persistent kernel of the bf16 path; it returns STM_ERR_UNSUPPORTED for shapes that kernel does
+ * not take (fewer than 4096 rows, n not a multiple of 8, fp32 output). */
+int stm_quantize_e4m3_1x128_pow2(const void* x, int dtype, int64_t rows, int64_t cols, uint8_t* codes_out,
+                                 float* scales_by_block_out, stm_stream_t stream);
+int stm_grouped_gemm_fp8_pow2(const uint8_t* a_codes, const float* a_scales_by_block, const uint8_t* b_codes,
+                              const float* b_scales_by_block, void* c, const int32_t* offsets, int n_groups,
+                              int64_t m_cap, int n, int k, int out_dtype, void* workspace, size_t workspace_bytes,
+                              stm_stream_t stream);
 int stm_grouped_gemm_fp8(const uint8_t* a_codes, const float* a_scales, const uint8_t* b_codes, const float* b_scales,
                          void* c, const int32_t* offsets, int n_groups, int64_t m_cap, int n, int k, int out_dtype,
                          void* workspace, size_t workspace_bytes, stm_stream_t stream);

@@ -572,10 +572,11 @@ def e4m3_round(x: torch.Tensor) -> torch.Tensor:
     return code.to(torch.uint8)
 
 
-def quantize_e4m3_1x128(x: torch.Tensor, block: int = 128):
+def quantize_e4m3_1x128(x: torch.Tensor, block: int = 128, pow2: bool = False):
     """Per-row, per-``block``-column scaling: ``scale = amax/448`` (1.0 for an all-zero
     block), codes = round_e4m3(x/scale).  Returns ``(codes uint8 [R,C], scales fp32
-    [R, ceil(C/block)])``."""
+    [R, ceil(C/block)])``.  ``pow2``: the scale is raised to the next power of two (at least
+    the smallest normal fp32), the form a block-scaled matrix instruction applies in hardware."""
     R, C = x.shape
     nb = (C + block - 1) // block
     xf = x.float()
@@ -585,6 +586,10 @@ def quantize_e4m3_1x128(x: torch.Tensor, block: int = 128):
     xb = xf.reshape(R, nb, block)
     amax = xb.abs().amax(2)
     scale = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax))
+    if pow2:
+        mant, expo = torch.frexp(scale)  # scale = mant * 2^expo, mant in [0.5, 1)
+        expo = torch.where(mant == 0.5, expo - 1, expo).clamp(min=-126)
+        scale = torch.ldexp(torch.ones_like(scale), expo)
     q = e4m3_round((xb / scale.unsqueeze(2)).reshape(R, nb * block))[:, :C]
     return q.contiguous(), scale
 

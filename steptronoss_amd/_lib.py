@@ -65,7 +65,9 @@ SIGNATURES = {
     "stm_slot_values_to_rows": (I, [P, I, P, L, P, L, P]),
     "stm_row_parts_to_slots": (I, [P, I, P, L, L, P, I, P]),
     "stm_quantize_e4m3_1x128": (I, [P, I, L, L, P, P, P]),
+    "stm_quantize_e4m3_1x128_pow2": (I, [P, I, L, L, P, P, P]),
     "stm_grouped_gemm_fp8": (I, [P, P, P, P, P, P, I, L, I, I, I, P, Z, P]),
+    "stm_grouped_gemm_fp8_pow2": (I, [P, P, P, P, P, P, I, L, I, I, I, P, Z, P]),
     "stm_swiglu_fwd": (I, [P, P, L, L, P, I, F, I, P]),
     "stm_swiglu_bwd": (I, [P, P, P, L, L, P, I, F, I, P]),
     "stm_router_workspace_bytes": (Z, [L, I]),

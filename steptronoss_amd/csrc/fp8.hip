@@ -27,6 +27,18 @@ __device__ __forceinline__ uint32_t e4m3_code(float v) {
   return sign | code;
 }
 
+// The scale of a block whose largest magnitude is amax: amax / 448, or (POW2) the smallest power
+// of two that is not below it, which the block-scaled MFMA takes as an exponent byte.
+template <bool POW2>
+__device__ __forceinline__ float block_scale(float amax) {
+  if (!(amax > 0.f)) return 1.f;
+  const float s = amax / kE4m3Max;
+  if constexpr (!POW2) return s;
+  uint32_t b = __float_as_uint(s);
+  b = (b & 0x7fffffu) ? (b & 0x7f800000u) + 0x00800000u : (b & 0x7f800000u);
+  return __uint_as_float(b < 0x00800000u ? 0x00800000u : b);  // at least the smallest normal
+}
+
 // 16 lanes per (row, block), eight elements per lane (one 16-byte load of 16-bit inputs, one
 // 8-byte store of codes); a wavefront takes four blocks.  cols is a multiple of 8 here.
 template <typename T>
@@ -34,7 +46,9 @@ struct alignas(sizeof(T) * 8) In8 {
   T v[8];
 };
 
-template <typename T>
+// POW2: power-of-two scales, stored block-major (scales[b * rows + r]) for the GEMM that reads
+// them by row; otherwise scales[r * n_blocks + b].
+template <typename T, bool POW2>
 __global__ __launch_bounds__(256) void quantize_vec_kernel(const T* __restrict__ x, uint8_t* __restrict__ codes,
                                                            float* __restrict__ scales, int64_t rows, int64_t cols,
                                                            int64_t n_blocks) {
@@ -58,8 +72,8 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(const T* __restrict__
   for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[e]));
 #pragma unroll
   for (int off = 8; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, kWave));
-  const float scale = amax > 0.f ? amax / kE4m3Max : 1.f;
-  if (live && sub == 0) scales[r * n_blocks + b] = scale;
+  const float scale = block_scale<POW2>(amax);
+  if (live && sub == 0) scales[POW2 ? b * rows + r : r * n_blocks + b] = scale;
   if (in) {
     uint32_t lo = 0, hi = 0;
 #pragma unroll
@@ -72,7 +86,7 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(const T* __restrict__
 }
 
 // Any width / alignment: one wavefront per (row, block), two elements per lane.
-template <typename T>
+template <typename T, bool POW2>
 __global__ __launch_bounds__(256) void quantize_kernel(const T* __restrict__ x, uint8_t* __restrict__ codes,
                                                        float* __restrict__ scales, int64_t rows, int64_t cols,
                                                        int64_t n_blocks) {
@@ -84,22 +98,38 @@ __global__ __launch_bounds__(256) void quantize_kernel(const T* __restrict__ x, 
   float v0 = c0 < cols ? to_float(x[r * cols + c0]) : 0.f;
   float v1 = c0 + 1 < cols ? to_float(x[r * cols + c0 + 1]) : 0.f;
   const float amax = wave_max(fmaxf(fabsf(v0), fabsf(v1)));
-  const float scale = amax > 0.f ? amax / kE4m3Max : 1.f;
-  if (lane == 0) scales[r * n_blocks + b] = scale;
+  const float scale = block_scale<POW2>(amax);
+  if (lane == 0) scales[POW2 ? b * rows + r : r * n_blocks + b] = scale;
   if (c0 < cols) codes[r * cols + c0] = uint8_t(e4m3_code(v0 / scale));
   if (c0 + 1 < cols) codes[r * cols + c0 + 1] = uint8_t(e4m3_code(v1 / scale));
 }
 
-template <typename T>
+template <typename T, bool POW2>
 int quantize_typed(const void* x, uint8_t* codes, float* scales, int64_t rows, int64_t cols, hipStream_t s) {
   const int64_t n_blocks = (cols + kQBlock - 1) / kQBlock;
   const int64_t units = rows * n_blocks;
   const T* in = static_cast<const T*>(x);
   if (cols % 8 == 0 && aligned_to(x, sizeof(T) * 8) && aligned_to(codes, 8))
-    quantize_vec_kernel<T><<<unsigned((units + 15) / 16), 256, 0, s>>>(in, codes, scales, rows, cols, n_blocks);
+    quantize_vec_kernel<T, POW2><<<unsigned((units + 15) / 16), 256, 0, s>>>(in, codes, scales, rows, cols, n_blocks);
   else
-    quantize_kernel<T><<<unsigned((units + 3) / 4), 256, 0, s>>>(in, codes, scales, rows, cols, n_blocks);
+    quantize_kernel<T, POW2><<<unsigned((units + 3) / 4), 256, 0, s>>>(in, codes, scales, rows, cols, n_blocks);
   return launch_status();
+}
+
+template <bool POW2>
+int quantize_any(const void* x, int dtype, int64_t rows, int64_t cols, uint8_t* codes_out, float* scales_out,
+                 hipStream_t s) {
+  if (rows < 0 || cols < 0) return STM_ERR_ARG;
+  if (dtype < STM_F32 || dtype > STM_BF16) return STM_ERR_UNSUPPORTED;
+  if (rows == 0 || cols == 0) return STM_OK;
+  if (!x || !codes_out || !scales_out) return STM_ERR_ARG;
+  const int64_t units = rows * ((cols + kQBlock - 1) / kQBlock);
+  if (units > 0x7fffffffll * 4) return STM_ERR_UNSUPPORTED;
+  switch (dtype) {
+    case STM_F32: return quantize_typed<float, POW2>(x, codes_out, scales_out, rows, cols, s);
+    case STM_F16: return quantize_typed<f16_t, POW2>(x, codes_out, scales_out, rows, cols, s);
+    default: return quantize_typed<bf16_t, POW2>(x, codes_out, scales_out, rows, cols, s);
+  }
 }
 
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
@@ -234,19 +264,12 @@ extern "C" {
 
 int stm_quantize_e4m3_1x128(const void* x, int dtype, int64_t rows, int64_t cols, uint8_t* codes_out, float* scales_out,
                             stm_stream_t stream) {
-  using namespace stm;
-  if (rows < 0 || cols < 0) return STM_ERR_ARG;
-  if (dtype < STM_F32 || dtype > STM_BF16) return STM_ERR_UNSUPPORTED;
-  if (rows == 0 || cols == 0) return STM_OK;
-  if (!x || !codes_out || !scales_out) return STM_ERR_ARG;
-  const int64_t units = rows * ((cols + kQBlock - 1) / kQBlock);
-  if (units > 0x7fffffffll * 4) return STM_ERR_UNSUPPORTED;
-  hipStream_t s = as_stream(stream);
-  switch (dtype) {
-    case STM_F32: return quantize_typed<float>(x, codes_out, scales_out, rows, cols, s);
-    case STM_F16: return quantize_typed<f16_t>(x, codes_out, scales_out, rows, cols, s);
-    default: return quantize_typed<bf16_t>(x, codes_out, scales_out, rows, cols, s);
-  }
+  return stm::quantize_any<false>(x, dtype, rows, cols, codes_out, scales_out, stm::as_stream(stream));
+}
+
+int stm_quantize_e4m3_1x128_pow2(const void* x, int dtype, int64_t rows, int64_t cols, uint8_t* codes_out,
+                                 float* scales_by_block_out, stm_stream_t stream) {
+  return stm::quantize_any<true>(x, dtype, rows, cols, codes_out, scales_by_block_out, stm::as_stream(stream));
 }
 
 int stm_grouped_gemm_fp8(const uint8_t* a_codes, const float* a_scales, const uint8_t* b_codes, const float* b_scales,
@@ -271,6 +294,39 @@ int stm_grouped_gemm_fp8(const uint8_t* a_codes, const float* a_scales, const ui
     default: fp8_gemm_kernel<bf16_t><<<grid, 256, 0, s>>>(p); break;
   }
   return launch_status();
+}
+
+int stm_grouped_gemm_fp8_pow2(const uint8_t* a_codes, const float* a_scales_by_block, const uint8_t* b_codes,
+                              const float* b_scales_by_block, void* c, const int32_t* offsets, int n_groups,
+                              int64_t m_cap, int n, int k, int out_dtype, void* workspace, size_t workspace_bytes,
+                              stm_stream_t stream) {
+  using namespace stm;
+  if (n_groups < 0 || m_cap < 0 || n < 0 || k < 0) return STM_ERR_ARG;
+  if (k % kQBlock != 0 || n_groups > 4096) return STM_ERR_UNSUPPORTED;
+  if (m_cap == 0 || n == 0 || n_groups == 0 || k == 0) return STM_ERR_UNSUPPORTED;  // the plain entry handles it
+  if (!a_codes || !a_scales_by_block || !b_codes || !b_scales_by_block || !c || !offsets || !workspace)
+    return STM_ERR_ARG;
+  if (!aligned_to(a_codes, 16) || !aligned_to(b_codes, 16) || !aligned_to(c, 16)) return STM_ERR_UNSUPPORTED;
+  if (workspace_bytes < stm_gemm_workspace_bytes(m_cap, n_groups)) return STM_ERR_WORKSPACE;
+  GemmArgs p{};
+  p.a = a_codes;
+  p.b = b_codes;
+  p.c = c;
+  p.offsets = offsets;
+  p.header = static_cast<const int32_t*>(workspace);
+  p.tiles = reinterpret_cast<const MTile*>(static_cast<const char*>(workspace) + 16);
+  p.n_groups = n_groups;
+  p.lda = k / 2;  // 16-bit units of two codes
+  p.ldb = k / 2;
+  p.ldc = n;
+  p.b_group = int64_t(n) * (k / 2);
+  p.n_j = n;
+  p.n_k = k / 2;
+  p.a_scales = a_scales_by_block;
+  p.b_scales = b_scales_by_block;
+  p.a_scale_rows = m_cap;
+  p.b_scale_rows = int64_t(n_groups) * n;
+  return launch_dma_fp8(out_dtype, p, offsets, n_groups, m_cap, workspace, as_stream(stream));
 }
 
 }  // extern "C"

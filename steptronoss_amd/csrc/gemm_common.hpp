@@ -66,6 +66,12 @@ struct GemmArgs {
   // per row: row_dot is fp32 [M, 2 * tiles_j].
   const float* row_scale;
   float* row_dot;
+  // fp8 (e4m3) operands, rows form: a and b hold codes (two per 16-bit unit: lda, ldb, n_k count
+  // units), one power-of-two scale per row and 128 codes, stored block-major:
+  // a_scales[kb * a_scale_rows + r], b_scales[kb * b_scale_rows + g * n_j + j].
+  const float* a_scales;
+  const float* b_scales;
+  int64_t a_scale_rows, b_scale_rows;
 };
 
 // Fused SwiGLU forms of the rows GEMM (gemm_mfma_dma.hip); STM_ERR_UNSUPPORTED when the shape does not fit.
@@ -73,6 +79,10 @@ int launch_dma_swiglu_fwd(int dtype, const GemmArgs& base, const int32_t* offset
                           void* ws, hipStream_t s);
 int launch_dma_swiglu_bwd(int dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap,
                           void* ws, hipStream_t s);
+
+// fp8 operands through the same pipeline (gemm_mfma_dma.hip): c = a * b[g]^T in bf16 / fp16.
+int launch_dma_fp8(int out_dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap, void* ws,
+                   hipStream_t s);
 
 // Enqueue the kernel that fills the table for tiles of height bm (defined in gemm_generic.hip).
 int build_tile_table(const int32_t* offsets, int n_groups, int bm, int64_t m_cap, void* table, hipStream_t stream);

@@ -199,11 +199,12 @@ struct TileState {
   uint32_t soff_b0;  // scalar offset of this wave's first B load of a stage at contraction step 0
   int col0;          // first output column of the tile (fused SwiGLU: first gate column)
   int row0;          // rows form: first row of the tile in the whole problem
+  int64_t brow0;     // rows form: row of the tile's first column in b seen as [G * n_j, k]
   int valid_i, valid_j, n_steps;
 };
 
 // What the epilogue does with the accumulators.
-enum Epilogue { kStore = 0, kSwigluFwd = 1, kSwigluBwd = 2, kAccumF32 = 3 };
+enum Epilogue { kStore = 0, kSwigluFwd = 1, kSwigluBwd = 2, kAccumF32 = 3, kStoreFp8 = 4 };
 
 // WAVES = 4: one wave per SIMD, 2 x 2 waves of 128 x 128 outputs each.
 // WAVES = 8: two waves per SIMD, 4 x 2 waves of 64 x 128 outputs each: while one wave of a SIMD
@@ -221,6 +222,11 @@ enum Epilogue { kStore = 0, kSwigluFwd = 1, kSwigluBwd = 2, kAccumF32 = 3 };
 //   d gate_up.
 // EPI = kAccumF32 (wgrad): the product is added to an fp32 buffer of the output's shape (a
 //   gradient accumulator) instead of being stored in T.
+// EPI = kStoreFp8 (C = A * W^T on e4m3 codes): the operands are seen as 16-bit units of two codes,
+//   so a stage of 64 units is one 128-code scale block and every address of the pipeline is
+//   unchanged; the products run on v_mfma_scale_f32_32x32x64_f8f6f4, which multiplies each
+//   operand by a power of two given as an exponent byte: the per-row, per-block scales go in
+//   there and the fp32 accumulators need no rescaling.  T is the output type.
 template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int kBK, int EPI>
 __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs p) {
   static_assert(kBK == 64 || kBK == 32, "contraction elements per stage");
@@ -228,6 +234,8 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
                 "fused SwiGLU epilogues: rows form, 8 waves");
   static_assert(EPI != kAccumF32 || (WAVES == 8 && WGRAD), "accumulation into an fp32 buffer: wgrad, 8 waves");
   static_assert(EPI != kSwigluFwd || !B_KM, "the fused forward reads W1 rows K-contiguous");
+  constexpr bool kFp8 = EPI == kStoreFp8;
+  static_assert(!kFp8 || (!A_KM && !B_KM && !WGRAD && WAVES == 8 && kBK == 64), "fp8: rows form, both operands K-contiguous");
   constexpr int kStages = (1 << kStagesBytesLog2) / ((BM + BN) * kBK * 2);
   constexpr int WROWS = WAVES / 2;                   // wave rows; two wave columns
   constexpr int TM = BM / 32 / WROWS, TN = BN / 64;  // 32x32 MFMA tiles per wave
@@ -300,6 +308,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     t.valid_j = (EPI == kSwigluFwd ? p.ffn : p.n_j) - j0;
     t.col0 = j0;
     t.row0 = 0;
+    t.brow0 = 0;
     t.c2 = nullptr;
     t.soff_b0 = 0;
     if constexpr (WGRAD) {
@@ -330,9 +339,10 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       n_k = p.n_k;
       t.valid_i = mt.rows;
       t.row0 = mt.row0;
+      t.brow0 = int64_t(mt.group) * p.n_j + j0;
       a += int64_t(mt.row0) * p.lda;
-      c += int64_t(mt.row0) * p.ldc + (EPI == kStore ? j0 : 0);
-      if constexpr (EPI != kStore) t.c2 = static_cast<T*>(p.c2) + int64_t(mt.row0) * p.ldc2;
+      c += int64_t(mt.row0) * p.ldc + (EPI == kStore || EPI == kStoreFp8 ? j0 : 0);
+      if constexpr (EPI != kStore && EPI != kStoreFp8) t.c2 = static_cast<T*>(p.c2) + int64_t(mt.row0) * p.ldc2;
       a_bytes = uint32_t(int64_t(mt.rows) * p.lda * 2);
       if constexpr (EPI == kSwigluFwd) {
         // the descriptor covers all 2*ffn rows of the expert's W1; this wave's 32 tile rows are
@@ -490,6 +500,92 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     using CL = std::integral_constant<int, kLoads>;
 
     const int n_steps = cur.n_steps;
+    if constexpr (kFp8) {
+      // One step = one 128-code scale block = two MFMAs (64 codes each) per pair of sub-blocks.
+      // A lane feeds the MFMA 32 codes of its row: the 16-byte chunks 2h and 2h+1 (h = lane / 32)
+      // of the 64-byte half row; both operands use the same rule, so matching codes meet.
+      typedef int i32x8_t __attribute__((ext_vector_type(8)));
+      const uint32_t scale_bytes_a = uint32_t(p.a_scale_rows * (p.n_k / kBK) * 4);
+      const uint32_t scale_bytes_b = uint32_t(p.b_scale_rows * (p.n_k / kBK) * 4);
+      const __amdgpu_buffer_rsrc_t rsrc_sa =
+          __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.a_scales), 0, int(scale_bytes_a), 0x00020000);
+      const __amdgpu_buffer_rsrc_t rsrc_sb =
+          __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.b_scales), 0, int(scale_bytes_b), 0x00020000);
+      // the scales of block kb as raw floats: a power of two 2^e is the float with exponent
+      // field e + 127, which is the byte the MFMA wants (rows past the operand read 0: 2^-127)
+      auto load_scales = [&](int kb, uint32_t (&sa)[TM], uint32_t (&sb)[TN]) {
+        const uint32_t soff_a = __builtin_amdgcn_readfirstlane(uint32_t((int64_t(kb) * p.a_scale_rows + cur.row0) * 4));
+        const uint32_t soff_b = __builtin_amdgcn_readfirstlane(uint32_t((int64_t(kb) * p.b_scale_rows + cur.brow0) * 4));
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          sa[i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sa, uint32_t((WROWS * i + wave_row) * 32 + tl % 32) * 4u,
+                                                       soff_a, 0);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          sb[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sb, uint32_t(wave_j + j * 32 + tl % 32) * 4u, soff_b, 0);
+      };
+      // (the exponent bytes are taken right after the wait that precedes the barrier, before any
+      // new load is issued: the compiler's own wait for these values then costs nothing)
+      auto take_exponents = [&](const uint32_t (&ra)[TM], const uint32_t (&rb)[TN], int (&sa)[TM], int (&sb)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          sa[i] = int(ra[i] >> 23);
+          asm volatile("" : "+v"(sa[i]));
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          sb[j] = int(rb[j] >> 23);
+          asm volatile("" : "+v"(sb[j]));
+        }
+      };
+      auto read_codes = [&](const unsigned char* tile, int r0, int f) {
+        const int r = r0 + tl % 32;
+        const int sw = (r >> 1) & 7;
+        const int c = f * 4 + (tl / 32) * 2;
+        const uint4 lo = *reinterpret_cast<const uint4*>(tile + r * 128 + ((c ^ sw) * 16));
+        const uint4 hi = *reinterpret_cast<const uint4*>(tile + r * 128 + (((c + 1) ^ sw) * 16));
+        i32x8_t v;
+        v[0] = int(lo.x), v[1] = int(lo.y), v[2] = int(lo.z), v[3] = int(lo.w);
+        v[4] = int(hi.x), v[5] = int(hi.y), v[6] = int(hi.z), v[7] = int(hi.w);
+        return v;
+      };
+      int sa_cur[TM], sb_cur[TN];
+      uint32_t sa_next[TM], sb_next[TN];
+      load_scales(0, sa_next, sb_next);
+      take_exponents(sa_next, sb_next, sa_cur, sb_cur);
+      for (int step = 0; step < n_steps; ++step) {
+        load_scales(step + 1 < n_steps ? step + 1 : step, sa_next, sb_next);  // (past the last block: a re-read)
+        const unsigned char* ta = smem + c_slot;
+        const unsigned char* tb = ta + PlanA::kStageBytes;
+        int loads_done = kEarly;
+#pragma unroll
+        for (int f = 0; f < 2; ++f) {
+          i32x8_t qa[AR];
+#pragma unroll
+          for (int i = 0; i < ATM; ++i) qa[i] = read_codes(ta, (WROWS * i + wave_row) * 32, f);
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            const i32x8_t qb = read_codes(tb, wave_j + j * 32, f);
+#pragma unroll
+            for (int i = 0; i < ATM; ++i)  // operands swapped, as everywhere: a lane owns output row lane % 32
+              acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(qb, qa[i], acc[i][j], 0, 0, 0, sb_cur[j], 0,
+                                                                          sa_cur[i]);
+            if (loads_done < kLoads) issue_one_load(loads_done++);
+          }
+        }
+#pragma unroll
+        for (int li = kEarly; li < kLoads; ++li)
+          if (li >= loads_done) issue_one_load(li);
+        advance_loads();
+        // the next stage has landed (my part) and my reads of this one are done; after the barrier
+        // both hold for the workgroup, and this stage's slot can be refilled
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        c_slot = (c_slot + kStageBytes) & (kStages * kStageBytes - 1);
+        take_exponents(sa_next, sb_next, sa_cur, sb_cur);
+        issue_loads(std::integral_constant<int, 0>{}, std::integral_constant<int, kEarly>{});
+      }
+    } else
     for (int step = 0; step < n_steps; ++step) {
       if constexpr (kBK == 64) {
         slice(0, true, c_slot, 1, CE{}, CM{});
@@ -615,7 +711,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
             }
           }
         }
-      } else if constexpr (EPI == kStore) {
+      } else if constexpr (EPI == kStore || EPI == kStoreFp8) {
 #pragma unroll
         for (int i = 0; i < ATM; ++i) {
           const int row0 = (WROWS * i + wave_row) * 32;
@@ -911,6 +1007,25 @@ int launch_dma_swiglu_bwd(int dtype, const GemmArgs& base, const int32_t* offset
   p.tiles_j = (p.ffn + kDmaBN - 1) / kDmaBN;
   if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, false, true, false, 32, kSwigluBwd>(p, s);
   return launch<f16_t, kDmaBM, kDmaBN, false, true, false, 32, kSwigluBwd>(p, s);
+}
+
+// e4m3 operands (codes; lda, ldb, n_k in 16-bit units of two codes), power-of-two scales stored
+// block-major; c in bf16 or fp16.
+int launch_dma_fp8(int out_dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap, void* ws,
+                   hipStream_t s) {
+  GemmArgs p = base;
+  if (out_dtype != STM_BF16 && out_dtype != STM_F16) return STM_ERR_UNSUPPORTED;
+  if (p.n_k % 64 != 0 || p.n_j % 8 != 0 || m_cap < 4096) return STM_ERR_UNSUPPORTED;
+  if (int64_t(p.n_k) * p.ldb * 2 >= (int64_t(1) << 32) || int64_t(kDmaBM) * p.lda * 2 >= (int64_t(1) << 32))
+    return STM_ERR_UNSUPPORTED;
+  const int64_t n_kb = p.n_k / 64;
+  if (p.a_scale_rows * n_kb * 4 >= (int64_t(1) << 31) || p.b_scale_rows * n_kb * 4 >= (int64_t(1) << 31))
+    return STM_ERR_UNSUPPORTED;
+  const int st = build_tile_table(offsets, n_groups, kDmaBM, m_cap, ws, s);
+  if (st != STM_OK) return st;
+  p.tiles_j = (p.n_j + kDmaBN - 1) / kDmaBN;
+  if (out_dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, false, false, false, 64, kStoreFp8>(p, s);
+  return launch<f16_t, kDmaBM, kDmaBN, false, false, false, 64, kStoreFp8>(p, s);
 }
 
 // accumulate != 0: base.c is an fp32 buffer [G, P, Q] and the product is added to it.

@@ -30,6 +30,53 @@ def quantize_e4m3_1x128(x: torch.Tensor):
     return codes, scales
 
 
+def quantize_e4m3_1x128_pow2(x: torch.Tensor):
+    """``(codes uint8 [R, C], scales float32 [ceil(C/128), R])`` of a matrix (leading axes
+    flattened to ``R``): power-of-two scales, stored block-major, as ``grouped_gemm_fp8_pow2``
+    reads them."""
+    require_gpu(x)
+    xc = x.contiguous()
+    cols = xc.shape[-1]
+    rows = xc.numel() // max(cols, 1)
+    codes = torch.empty(xc.shape, device=x.device, dtype=torch.uint8)
+    scales = torch.empty(((cols + BLOCK - 1) // BLOCK, rows), device=x.device, dtype=torch.float32)
+    with torch.cuda.device(x.device):
+        call("stm_quantize_e4m3_1x128_pow2", ptr(xc), dtype_code(xc.dtype), rows, cols, ptr(codes), ptr(scales), stream())
+    return codes, scales
+
+
+def grouped_gemm_fp8_pow2(a_codes, a_scales, b_codes, b_scales, batch_sizes, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """As :func:`grouped_gemm_fp8` on the operands of :func:`quantize_e4m3_1x128_pow2`
+    (``a_scales`` ``[K/128, M]``, ``b_scales`` ``[K/128, G*N]``): the scales go into the
+    block-scaled matrix instruction, the kernel is the persistent one of the bf16 path.
+    ``out_dtype`` bf16 or fp16; at least 4096 rows (``NotImplementedError`` otherwise)."""
+    from steptronoss_amd.model.utils.moe_utils import _gemm_workspace, _group_offsets
+
+    dev = require_gpu(a_codes, b_codes, a_scales, b_scales)
+    if a_codes.dtype != torch.uint8 or b_codes.dtype != torch.uint8:
+        raise TypeError("codes must be uint8 tensors")
+    if a_codes.dim() != 2 or b_codes.dim() != 3 or a_codes.shape[1] != b_codes.shape[2]:
+        raise ValueError("a must be [M, K] and b [G, N, K]")
+    m_cap, k = a_codes.shape
+    n_groups, n, _ = b_codes.shape
+    if k % BLOCK:
+        raise ValueError("the contraction length must be a multiple of 128")
+    if a_scales.shape != (k // BLOCK, m_cap) or b_scales.shape != (k // BLOCK, n_groups * n):
+        raise ValueError("scales must be [K/128, M] and [K/128, G*N]")
+    with torch.cuda.device(dev):
+        offsets = _group_offsets(batch_sizes, dev)
+        out = torch.zeros((m_cap, n), device=dev, dtype=out_dtype)
+        ws = _gemm_workspace(m_cap, n_groups, dev)
+        ok = _lib.try_call(
+            "stm_grouped_gemm_fp8_pow2", ptr(a_codes.contiguous()), ptr(a_scales.contiguous().float()),
+            ptr(b_codes.contiguous()), ptr(b_scales.contiguous().float()), ptr(out), ptr(offsets), n_groups, m_cap, n, k,
+            dtype_code(out_dtype), ptr(ws), ws.numel(), stream(),
+        )  # fmt: skip
+    if not ok:
+        raise NotImplementedError("grouped_gemm_fp8_pow2: shape or output type outside the persistent kernel")
+    return out
+
+
 def grouped_gemm_fp8(a_codes, a_scales, b_codes, b_scales, batch_sizes, out_dtype=torch.bfloat16) -> torch.Tensor:
     """``out[rows of g] = dequant(a)[rows of g] @ dequant(b[g])^T`` with ``a`` ``[M, K]`` and ``b``
     ``[G, N, K]`` quantised along ``K`` (a multiple of 128); products and sums in fp32."""

@@ -89,3 +89,73 @@ def test_fp8_forward_and_dgrad_of_an_expert_layer():
     assert rel_l2(y, O.grouped_gemm(x.float(), w1.float(), bs, trans_b=True)) <= QUANT_NOISE_TOL
     ref_dx, _ = O.grouped_gemm_grads(x.float(), w1.float(), bs, True, dy.float())
     assert rel_l2(dx, ref_dx) <= QUANT_NOISE_TOL
+
+
+# ----- power-of-two scales and the block-scaled matrix instruction (persistent kernel)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,cols", [(7, 128), (33, 384), (5, 200), (64, 1024)])
+def test_pow2_quantiser_matches_oracle_bit_for_bit(rows, cols, dtype):
+    from steptronoss_amd.model.utils.fp8 import quantize_e4m3_1x128_pow2
+
+    gen = torch.Generator().manual_seed(rows * 1000 + cols + 1)
+    x = (torch.randn(rows, cols, generator=gen) * torch.logspace(-4, 2, rows).unsqueeze(1)).to(dtype)
+    x[0, :128] = 0  # an all-zero block
+    x[2, :128] = 0
+    x[2, 3] = 448.0  # amax / 448 is a power of two already: the scale stays 1
+    q_ref, s_ref = O.quantize_e4m3_1x128(x.float(), pow2=True)
+    q, s = quantize_e4m3_1x128_pow2(x.to(DEV))
+    assert s.shape == (s_ref.shape[1], rows)
+    assert torch.equal(s.cpu().t(), s_ref)
+    assert float(s_ref[2, 0]) == 1.0
+    mant, _ = torch.frexp(s.cpu())
+    assert bool((mant == 0.5).all()), "scales must be powers of two"
+    assert torch.equal(q.cpu(), q_ref)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize(
+    "sizes,k,n",
+    [
+        ([1000, 0, 37, 2500, 300, 900], 256, 192),  # ragged groups, an empty one, a partly used column tile
+        ([4096, 256], 128, 72),  # one block of contraction, a narrow output
+        ([513, 2047, 1536, 1], 896, 256),  # seven blocks
+    ],
+)
+def test_grouped_gemm_fp8_pow2(sizes, k, n, out_dtype):
+    from steptronoss_amd.model.utils.fp8 import grouped_gemm_fp8, grouped_gemm_fp8_pow2, quantize_e4m3_1x128_pow2
+
+    gen = torch.Generator().manual_seed(23)
+    m, G = sum(sizes), len(sizes)
+    a = (torch.randn(m, k, generator=gen) * torch.logspace(-2, 1, m).unsqueeze(1)).bfloat16()  # scales differ by row
+    w = (torch.randn(G, n, k, generator=gen) * 0.05).bfloat16()
+    aq, as_ = quantize_e4m3_1x128_pow2(a.to(DEV))
+    wq, ws = quantize_e4m3_1x128_pow2(w.to(DEV))
+    out = grouped_gemm_fp8_pow2(aq, as_, wq, ws, torch.tensor(sizes), out_dtype=out_dtype)
+    # exact arithmetic on the quantised operands.  The matrix instruction aligns the 64 products of
+    # a step to a common exponent before adding them (about 12 bits relative to the largest), so
+    # the bar is looser than for the fp32-accumulating kernel but far below the quantisation noise.
+    a_dq = O.dequantize_e4m3_1x128(aq.cpu(), as_.cpu().t().contiguous())
+    w_dq = O.dequantize_e4m3_1x128(wq.cpu().reshape(G * n, k), ws.cpu().t().contiguous()).reshape(G, n, k)
+    ref_q = O.grouped_gemm(a_dq, w_dq, torch.tensor(sizes), trans_b=True)
+    assert rel_l2(out, ref_q) <= 4e-3
+    # the plain fp8 kernel on the same operands (scales in its row-major layout)
+    plain = grouped_gemm_fp8(aq, as_.t().contiguous(), wq, ws.t().contiguous().reshape(G, n, -1), torch.tensor(sizes),
+                             out_dtype=out_dtype)  # fmt: skip
+    assert rel_l2(out, plain.float()) <= 4e-3
+    # against the unquantised product: quantisation noise (power-of-two scales use the e4m3 range a
+    # little less well than amax/448)
+    ref = O.grouped_gemm(a.float(), w.float(), torch.tensor(sizes), trans_b=True)
+    assert rel_l2(out, ref) <= QUANT_NOISE_TOL
+    rows_used = sum(sizes)
+    assert bool(torch.isfinite(out[:rows_used].float()).all())
+
+
+def test_grouped_gemm_fp8_pow2_declines_small_problems():
+    from steptronoss_amd.model.utils.fp8 import grouped_gemm_fp8_pow2, quantize_e4m3_1x128_pow2
+
+    a = torch.randn(64, 128, device=DEV).bfloat16()
+    w = torch.randn(2, 16, 128, device=DEV).bfloat16()
+    aq, as_ = quantize_e4m3_1x128_pow2(a)
+    wq, ws = quantize_e4m3_1x128_pow2(w)
+    with pytest.raises(NotImplementedError):
+        grouped_gemm_fp8_pow2(aq, as_, wq, ws, torch.tensor([30, 34]))
