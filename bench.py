@@ -46,7 +46,10 @@ WORKLOADS = {
     "c2": dict(T=16384, H=2048, E=128, K=8, F=768, sigmoid=False, norm=True, n_group=1, topk_group=1, std=0.02),
     "c3": dict(T=16384, H=2048, E=128, K=8, F=768, sigmoid=False, norm=True, n_group=1, topk_group=1, std=0.02, zipf=1.2),
     "c4": dict(T=8192, H=7168, E=256, K=8, F=2048, sigmoid=True, norm=True, n_group=8, topk_group=4, std=0.006),
+    # c4's shapes on e4m3 operands, forward + dgrad of the expert FFN on the routed rows (run_fp8)
+    "c5": dict(T=8192, H=7168, E=256, K=8, F=2048, sigmoid=True, norm=True, n_group=8, topk_group=4, std=0.006, dtype="fp8_e4m3"),
 }
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA
 
 
 def zipf_logit_bias(E, s, gen):
@@ -116,6 +119,115 @@ def cpu_baseline(cfg, seed, threads):
     }
 
 
+def cpu_baseline_fwd_dgrad(cfg, seed, threads):
+    """The expert FFN forward + input gradient (what the fp8 workload times) with the oracle on
+    CPU tensors, fp32, on a bounded sample: 32 of the experts at 256 rows each."""
+    from oracle import moe_oracle as O
+
+    torch.set_num_threads(threads)
+    H, F = cfg["H"], cfg["F"]
+    E, rows_per = 32, 256
+    gen = torch.Generator().manual_seed(seed)
+    x = (torch.randn(E * rows_per, H, generator=gen) * cfg["std"]).bfloat16().float().requires_grad_(True)
+    w1 = (torch.randn(E, 2 * F, H, generator=gen) * cfg["std"]).bfloat16().float()
+    w2 = (torch.randn(E, H, F, generator=gen) * cfg["std"]).bfloat16().float()
+    go = torch.randn(E * rows_per, H, generator=gen)
+    sizes = torch.full((E,), rows_per, dtype=torch.int64)
+    flops = 4.0 * E * rows_per * H * 3 * F
+    times = []
+    for _ in range(3):
+        x.grad = None
+        t0 = time.perf_counter()
+        y = O.grouped_gemm(O.swiglu(O.grouped_gemm(x, w1, sizes, trans_b=True)), w2, sizes, trans_b=True)
+        y.backward(go)
+        times.append(time.perf_counter() - t0)
+        if sum(times) > 12.0:
+            break
+    best = min(times)
+    return {
+        "value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": f"{E} of {cfg['E']} experts at {rows_per} rows each, fp32, forward + input gradient, best of "
+        f"{len(times)} passes, {best * 1e3:.0f} ms per pass",
+    }  # fmt: skip
+
+
+def run_fp8(args, cfg):
+    """Workload c5: the expert FFN of c4 on e4m3 operands (weights quantised once, activations on the
+    way into each GEMM), forward + dgrad over the rows the seeded router sends to each expert."""
+    from steptronoss_amd.model.common.moe_block import forward_router
+    from steptronoss_amd.model.utils.fp8 import Fp8ExpertFFN
+    from steptronoss_amd.model.utils.moe_utils import histogram, index_compute, moe_scatter
+    from steptronoss_amd.profiling import KernelTimer
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    bf16_cfg = dict(cfg, dtype="bf16")
+    x, w1, w2, logits, go = make_inputs(bf16_cfg, args.seed, dev)
+    T, H, E, K, F = cfg["T"], cfg["H"], cfg["E"], cfg["K"], cfg["F"]
+    N = T * K
+    ids, _w, _aux, _h = forward_router(
+        logits, K, use_sigmoid=cfg["sigmoid"], norm_expert_weight=cfg["norm"], n_group=cfg["n_group"],
+        topk_group=cfg["topk_group"],
+    )  # fmt: skip
+    sizes = histogram(ids, E)
+    pos = index_compute(ids, sizes)
+    rows = moe_scatter(x, pos).contiguous()
+    grad_rows = moe_scatter(go, pos).contiguous()
+    sizes = sizes.to(torch.int64)
+    ffn = Fp8ExpertFFN(w1, w2)
+    del w1, w2, x, go, logits
+    torch.cuda.empty_cache()
+
+    def step():
+        y, gate_up = ffn.forward_rows(rows, sizes)
+        return ffn.dgrad_rows(grad_rows, gate_up, sizes), y
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    with KernelTimer() as kt:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    flops = 4.0 * N * H * 3 * F
+    timing = kt.summary()
+    gemm = timing["stm_grouped_gemm_fp8_pow2"]
+    achieved = (flops / 4.0) / (gemm["avg_us"] * 1e-6) / 1e12
+    quant = timing["stm_quantize_e4m3_1x128_pow2"]
+    quant_bytes = (N * H * 3 + N * 2 * F * 3 + N * F * 3 + N * H * 3) / 4.0  # bf16 in, codes out, mean of the four
+    result = {
+        "metric": METRIC, "value": flops / (ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3", "data": "synthetic",
+        "config": {
+            "workload": f"c5: expert FFN of the c4 layer (T={T} H={H} E={E} top-{K} F={F}) on e4m3 operands with one "
+            "power-of-two scale per row and 128 elements, bf16 outputs; forward + dgrad over the routed rows "
+            "(weights quantised once, activations on the way into each GEMM)",
+            "tokens": T, "hidden": H, "experts": E, "top_k": K, "expert_ffn": F, "seed": args.seed,
+        },
+        "frac_of_mfma_peak": flops / (ms_per_step * 1e-3) / 1e12 / PEAK_FP8_TFLOPS,
+        "roofline": {
+            "bound": "mfma", "kernel": "persistent_gemm_kernel, e4m3 operands on v_mfma_scale_f32_32x32x64_f8f6f4",
+            "achieved": achieved, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_FP8_TFLOPS,
+            "traffic": None, "flops_per_launch": flops / 4.0, "avg_launch_us": gemm["avg_us"],
+            "launches_per_step": gemm["calls"] / args.steps,
+        },
+        "bandwidth": {
+            "quantize": {
+                "GB/s": quant_bytes / (quant["avg_us"] * 1e-6) / 1e9, "avg_us": quant["avg_us"], "bytes": quant_bytes,
+                "frac_of_hbm_peak": quant_bytes / (quant["avg_us"] * 1e-6) / 1e9 / PEAK_HBM_GBPS,
+            },
+        },
+        "entry_avg_us": {name: round(t["avg_us"], 1) for name, t in sorted(timing.items())},
+    }  # fmt: skip
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_fwd_dgrad(cfg, args.seed, min(os.cpu_count() or 1, 16))
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -143,6 +255,9 @@ def main():
     from steptronoss_amd.profiling import KernelTimer
 
     cfg = WORKLOADS[args.workload]
+    if cfg.get("dtype") == "fp8_e4m3":
+        run_fp8(args, cfg)
+        return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     x, w1, w2, logits, go = make_inputs(cfg, args.seed, dev)

@@ -4,7 +4,9 @@ The reference has no fp8 path (its grouped GEMMs run in the activations' dtype, 
 steptronoss/model/utils/moe_utils.py:423-453); this module serves the fp8 configuration of the
 benchmark: quantise activations and weights with one fp32 scale per row per 128 contraction
 elements, then ``grouped_gemm_fp8`` for the forward product and, on the transposed weights,
-for dgrad.
+for dgrad.  The ``_pow2`` pair does the same with power-of-two scales, which the block-scaled
+matrix instruction of gfx950 applies in hardware; :class:`Fp8ExpertFFN` strings the pieces into the
+forward and dgrad of an expert FFN.
 """
 
 from __future__ import annotations
@@ -103,6 +105,48 @@ def grouped_gemm_fp8(a_codes, a_scales, b_codes, b_scales, batch_sizes, out_dtyp
             dtype_code(out_dtype), ptr(ws), ws.numel(), stream(),
         )  # fmt: skip
     return out
+
+
+class Fp8ExpertFFN:
+    """The expert FFN on e4m3 operands, forward and dgrad (the fp8 benchmark configuration; weight
+    gradients stay with the bf16 path).  Weights are quantised once, in both orientations:
+    along their own contraction axis for the forward and, transposed, along the other one for
+    dgrad.  Activations are quantised on the way into each GEMM; GEMM outputs are bf16 / fp16.
+
+    ``rows`` are already in expert order (``moe_scatter``'s output); ``batch_sizes`` are the
+    rows per expert.
+    """
+
+    def __init__(self, w1: torch.Tensor, w2: torch.Tensor, swiglu_limit=None):
+        self.n_experts, two_f, self.hidden = w1.shape
+        self.ffn = two_f // 2
+        self.limit = swiglu_limit
+        self.w1_q, self.w1_s = quantize_e4m3_1x128_pow2(w1)  # [E, 2F, H] along H
+        self.w2_q, self.w2_s = quantize_e4m3_1x128_pow2(w2)  # [E, H, F] along F
+        self.w1t_q, self.w1t_s = quantize_e4m3_1x128_pow2(w1.transpose(1, 2).contiguous())  # [E, H, 2F] along 2F
+        self.w2t_q, self.w2t_s = quantize_e4m3_1x128_pow2(w2.transpose(1, 2).contiguous())  # [E, F, H] along H
+
+    def forward_rows(self, rows: torch.Tensor, batch_sizes: torch.Tensor):
+        """``y = swiglu(rows @ w1^T) @ w2^T`` per expert; returns ``(y, gate_up)``."""
+        from steptronoss_amd.model.common.feed_forward import swiglu_fwd_rows
+
+        q, sc = quantize_e4m3_1x128_pow2(rows)
+        gate_up = grouped_gemm_fp8_pow2(q, sc, self.w1_q, self.w1_s, batch_sizes, out_dtype=rows.dtype)
+        with torch.cuda.device(rows.device):
+            h = swiglu_fwd_rows(gate_up, self.limit)
+        q, sc = quantize_e4m3_1x128_pow2(h)
+        return grouped_gemm_fp8_pow2(q, sc, self.w2_q, self.w2_s, batch_sizes, out_dtype=rows.dtype), gate_up
+
+    def dgrad_rows(self, grad_y: torch.Tensor, gate_up: torch.Tensor, batch_sizes: torch.Tensor) -> torch.Tensor:
+        """Gradient of the rows given the gradient of ``y`` (the transposed weights as ``b``)."""
+        from steptronoss_amd.model.common.feed_forward import swiglu_bwd_rows
+
+        q, sc = quantize_e4m3_1x128_pow2(grad_y)
+        grad_h = grouped_gemm_fp8_pow2(q, sc, self.w2t_q, self.w2t_s, batch_sizes, out_dtype=grad_y.dtype)
+        with torch.cuda.device(grad_y.device):
+            grad_gate_up = swiglu_bwd_rows(gate_up, grad_h, self.limit)
+        q, sc = quantize_e4m3_1x128_pow2(grad_gate_up)
+        return grouped_gemm_fp8_pow2(q, sc, self.w1t_q, self.w1t_s, batch_sizes, out_dtype=grad_y.dtype)
 
 
 def _keepalive():  # the library handle, for callers that only import this module

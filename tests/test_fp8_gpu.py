@@ -159,3 +159,29 @@ def test_grouped_gemm_fp8_pow2_declines_small_problems():
     wq, ws = quantize_e4m3_1x128_pow2(w)
     with pytest.raises(NotImplementedError):
         grouped_gemm_fp8_pow2(aq, as_, wq, ws, torch.tensor([30, 34]))
+
+
+def test_fp8_expert_ffn_forward_and_dgrad_against_the_fp32_layer():
+    """Two chained fp8 GEMMs each way: every GEMM adds the e4m3 noise of its two operands
+    (about 3.6 % each, see the top of this file), so the layer's output and input gradient carry
+    about sqrt(2) times that; pinned below 7.5 % so that a real error still fails."""
+    from steptronoss_amd.model.utils.fp8 import Fp8ExpertFFN
+
+    gen = torch.Generator().manual_seed(31)
+    sizes = [1500, 0, 900, 1700, 300]
+    E, H, Fh = len(sizes), 256, 384
+    m = sum(sizes)
+    rows = (torch.randn(m, H, generator=gen) * 0.5).bfloat16()
+    w1 = (torch.randn(E, 2 * Fh, H, generator=gen) * 0.1).bfloat16()
+    w2 = (torch.randn(E, H, Fh, generator=gen) * 0.1).bfloat16()
+    gy = torch.randn(m, H, generator=gen).bfloat16()
+    bs = torch.tensor(sizes)
+    ffn = Fp8ExpertFFN(w1.to(DEV), w2.to(DEV))
+    y, gate_up = ffn.forward_rows(rows.to(DEV), bs)
+    gx = ffn.dgrad_rows(gy.to(DEV), gate_up, bs)
+    xr = rows.float().requires_grad_(True)
+    ref = O.grouped_gemm(O.swiglu(O.grouped_gemm(xr, w1.float(), bs, trans_b=True)), w2.float(), bs, trans_b=True)
+    ref.backward(gy.float())
+    assert rel_l2(y, ref) <= 7.5e-2
+    assert rel_l2(gx, xr.grad) <= 7.5e-2
+    assert rel_l2(y, ref) >= 1e-3  # it is an fp8 result, not the bf16 path by another name
