@@ -27,7 +27,8 @@ group-limited top-k    PARITY UNPINNED AGAINST THE REFERENCE (it has no such
                        routing); reduction n_group=1 => forward_router, python loop
 fp8 e4m3 quantiser     PARITY UNPINNED AGAINST THE REFERENCE (it has no fp8 MoE
                        path); exhaustive 256-code decode table, round trip,
-                       saturation
+                       saturation; the power-of-two scale form by hand-worked
+                       blocks (amax 448 -> 1, 449 -> 2, 3 -> 2^-7, tiny -> 2^-126)
 TE-style permute       brute-force expectations of tests/test_permute_utils.py
 update_router_balance  closed form on a hand-worked vector (over / under / at the
 _bias                  mean), sign symmetry

@@ -248,6 +248,26 @@ def test_quantize_1x128_round_trip():
     assert float((back - x).norm() / x.norm()) < 0.04
 
 
+def test_quantize_1x128_power_of_two_scales():
+    # hand-worked blocks: the scale is the smallest power of two >= amax / 448, never below 2^-126
+    x = torch.zeros(5, 128)
+    x[0, 0], x[1, 7], x[2, 3], x[3, 100] = 448.0, -449.0, 3.0, 1e-40
+    q, s = O.quantize_e4m3_1x128(x, pow2=True)
+    assert s.flatten().tolist() == [1.0, 2.0, 2.0**-7, 2.0**-126, 1.0]
+    assert int(q[0, 0]) == 0x7E and int(q[1, 7]) == 0xF6  # 448 -> largest code; -449/2 = -224.5 -> -224 (1.75 * 2^7)
+    assert int(q[2, 3]) == 0x7C  # 3 * 128 = 384 = 1.5 * 2^8
+    # against the plain form: never a smaller scale, less than twice as large, same decoded values to 2^-3 relative
+    g = torch.Generator().manual_seed(8)
+    y = torch.randn(9, 384, generator=g) * torch.logspace(-3, 2, 9).unsqueeze(1)
+    _, s_plain = O.quantize_e4m3_1x128(y)
+    q2, s2 = O.quantize_e4m3_1x128(y, pow2=True)
+    assert bool((s2 >= s_plain).all()) and bool((s2 < 2 * s_plain).all())
+    mant, _ = torch.frexp(s2)
+    assert bool((mant == 0.5).all())
+    back = O.dequantize_e4m3_1x128(q2, s2)
+    assert float((back - y).norm() / y.norm()) < 0.045
+
+
 # ----- TE-style helpers: reference tests/test_permute_utils.py -------------------------
 def _mask_expected(routing_map):
     T, E = routing_map.shape
