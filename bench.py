@@ -74,7 +74,14 @@ def make_inputs(cfg, seed, device):
         w2[e] = (torch.randn(H, F, generator=gen, device=device) * cfg["std"]).to(bf)
     logits = torch.randn(T, E, generator=gen, device=device)
     if "zipf" in cfg:
-        logits = logits + zipf_logit_bias(E, cfg["zipf"], torch.Generator().manual_seed(seed)).to(device)
+        # the skewed workload's logits come from a host generator, so that its per-expert loads are
+        # the same on every machine: a few experts above ten times the mean, at least one with none
+        host = torch.Generator().manual_seed(seed)
+        bias = zipf_logit_bias(E, cfg["zipf"], host)
+        host_logits = torch.randn(T, E, generator=host) + bias
+        loads = torch.bincount(host_logits.topk(cfg["K"], dim=1).indices.reshape(-1), minlength=E)
+        assert int(loads.max()) > 10 * T * cfg["K"] // E and int((loads == 0).sum()) >= 1, "c3 is not skewed enough"
+        logits = host_logits.to(device)
     go = torch.randn(T, H, generator=gen, device=device).to(bf)
     return x, w1, w2, logits, go
 

@@ -142,6 +142,22 @@ int stm_unpermute_bwd_scaled(const void* grad_out, const void* in, const void* p
                              int64_t hidden, int64_t n_in_rows, int dtype, uint8_t* written_or_null, int has_scale,
                              float scale, stm_stream_t stream);
 
+/* The early-out of routed_grouped_ffn (moe_utils.py:230-232: with no routed slot at all the op
+ * returns x * token_weights.sum()) decided on the device: n_routed is a device word (offsets[E]
+ * of stm_route_plan); the kernels leave at once unless it is zero, so a caller enqueues them
+ * after the combine (forward) and after the gradients (backward) with no host read-back.
+ *   forward : out[t,:] = round(x[t,:] * sum(weights)), then "* scale" and "+ addend" as in
+ *             stm_unpermute_fwd_epilogue;
+ *   backward: grad_x = (grad_out [* scale]) * sum(weights), grad_weight[s] = <grad_out [* scale], x>
+ *             for every slot (either output may be NULL).
+ * sum(weights) is rounded to the weights' element type, as the reference's tensor sum is. */
+int stm_nothing_routed_fwd(const int32_t* n_routed, const void* x, const void* weight, int weight_dtype, void* out,
+                           int64_t n_tokens, int top_k, int64_t hidden, int dtype, int has_scale, float scale,
+                           const void* addend_or_null, stm_stream_t stream);
+int stm_nothing_routed_bwd(const int32_t* n_routed, const void* grad_out, const void* x, const void* weight,
+                           int weight_dtype, void* grad_x_or_null, void* grad_weight_or_null, int64_t n_tokens,
+                           int top_k, int64_t hidden, int dtype, int has_scale, float scale, stm_stream_t stream);
+
 /* d input / d weight of moe_weighted_gather for ANY index, including one that names an input
  * row from several slots (the reference accumulates them with index_add_, moe_utils.py:302-305;
  * its own test uses such an index, tests/test_moe_utils.py:61-101).  Contributions to a row are
@@ -164,6 +180,10 @@ int stm_unpermute_bwd_general(const void* grad_out, const void* in, const void* 
  *   weight[i_j] * src[i_j / src_div], i_j = sorted_index[j]; fp32 sums in list order, rounded
  *   once; the deterministic form of the scatter_add_ of :201,:232. */
 size_t stm_sort_by_key_workspace_bytes(int64_t n, int64_t key_bound);
+/* out[j] = <a[j,:], b[j,:]> (fp32): the gradient of the per-row weight of a weighted scatter-add,
+ * i.e. of merging_probs in moe_unpermute (permute_utils.py:196-201, 226-232). */
+int stm_row_dot(const void* a, const void* b, float* out, int64_t n_rows, int64_t hidden, int dtype,
+                stm_stream_t stream);
 int stm_sort_by_key(const void* keys, int keys_are_i64, int64_t n, int64_t key_bound, int32_t* sorted_key,
                     int32_t* sorted_index, int32_t* n_valid_out, void* workspace, size_t workspace_bytes,
                     stm_stream_t stream);

@@ -48,10 +48,13 @@ SIGNATURES = {
     "stm_unpermute_bwd": (I, [P, P, P, I, P, I, P, P, L, I, L, L, I, P, P]),
     "stm_unpermute_fwd_epilogue": (I, [P, P, I, P, I, P, L, I, L, L, I, I, F, P, P]),
     "stm_unpermute_bwd_scaled": (I, [P, P, P, I, P, I, P, P, L, I, L, L, I, P, I, F, P]),
+    "stm_nothing_routed_fwd": (I, [P, P, P, I, P, L, I, L, I, I, F, P, P]),
+    "stm_nothing_routed_bwd": (I, [P, P, P, P, I, P, P, L, I, L, I, I, F, P]),
     "stm_unpermute_bwd_general_workspace_bytes": (Z, [L, L]),
     "stm_unpermute_bwd_general": (I, [P, P, P, I, P, I, P, P, L, I, L, L, I, P, Z, P]),
     "stm_sort_by_key_workspace_bytes": (Z, [L, L]),
     "stm_sort_by_key": (I, [P, I, L, L, P, P, P, P, Z, P]),
+    "stm_row_dot": (I, [P, P, P, L, L, I, P]),
     "stm_gather_rows": (I, [P, P, I, P, L, L, L, P]),
     "stm_segment_sum_rows": (I, [P, P, P, L, L, P, I, P, L, L, I, P]),
     "stm_index_check": (I, [P, I, L, L, P, P, P]),

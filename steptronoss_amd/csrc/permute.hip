@@ -341,6 +341,85 @@ __global__ void row_parts_to_slots_kernel(const float* __restrict__ parts, int n
   out[s] = from_float<W>(sum);
 }
 
+// ---------------------------------------------------------------- row dot products
+// out[j] = <a[j,:], b[j,:]> in fp32, one wavefront per row (the gradient of a per-row weight).
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void row_dot_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                              float* __restrict__ out, int64_t n_rows, int64_t hidden) {
+  const int64_t j = int64_t(blockIdx.x) * (kRowThreads / kWave) + threadIdx.x / kWave;
+  if (j >= n_rows) return;
+  float acc = 0.f;
+  for (int64_t u = threadIdx.x % kWave; u < hidden; u += kWave) acc += to_float(a[j * hidden + u]) * to_float(b[j * hidden + u]);
+  acc = wave_sum(acc);
+  if (threadIdx.x % kWave == 0) out[j] = acc;
+}
+
+// ---------------------------------------------------------------- nothing routed
+// routed_grouped_ffn's early-out: with no routed slot at all the op is x * sum(weights).
+// The routed count is a device word, so the decision is taken here, not on the host: every
+// workgroup reads it and leaves at once unless it is zero.
+__device__ __forceinline__ float block_sum_1024(float v, float* shared) {
+  v = wave_sum(v);
+  if (threadIdx.x % kWave == 0) shared[threadIdx.x / kWave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < int(blockDim.x) / kWave; ++w) total += shared[w];  // same order in every thread
+  __syncthreads();
+  return total;
+}
+
+// sum of all weights, as the element type of the weights would hold it
+__device__ __forceinline__ float weights_total(const void* weight, int wdtype, int64_t n_slots, float* shared) {
+  float part = 0.f;
+  for (int64_t i = threadIdx.x; i < n_slots; i += blockDim.x) part += load_weight_any(weight, wdtype, i);
+  const float total = block_sum_1024(part, shared);
+  return wdtype == STM_F32 ? total : (wdtype == STM_F16 ? round_through<f16_t>(total) : round_through<bf16_t>(total));
+}
+
+template <typename T>
+__global__ __launch_bounds__(1024) void nothing_routed_fwd_kernel(const int32_t* __restrict__ n_routed,
+                                                                  const T* __restrict__ x,
+                                                                  const void* __restrict__ weight, int wdtype,
+                                                                  T* __restrict__ out, int64_t n_tokens, int top_k,
+                                                                  int64_t hidden, bool has_scale, float scale,
+                                                                  const T* __restrict__ addend) {
+  __shared__ float shared[1024 / kWave];
+  if (*n_routed != 0) return;
+  const float wsum = weights_total(weight, wdtype, n_tokens * top_k, shared);
+  const int64_t n = n_tokens * hidden;
+  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += int64_t(gridDim.x) * blockDim.x) {
+    float v = round_through<T>(to_float(x[i]) * wsum);
+    if (has_scale) v = round_through<T>(v * scale);
+    if (addend) v += to_float(addend[i]);
+    out[i] = from_float<T>(v);
+  }
+}
+
+// One workgroup: d x = d out * sum(weights), d weight[s] = <d out, x> for every slot.
+template <typename T>
+__global__ __launch_bounds__(1024) void nothing_routed_bwd_kernel(const int32_t* __restrict__ n_routed,
+                                                                  const T* __restrict__ go, const T* __restrict__ x,
+                                                                  const void* __restrict__ weight, int wdtype,
+                                                                  T* __restrict__ gx, void* __restrict__ gw,
+                                                                  int64_t n_tokens, int top_k, int64_t hidden,
+                                                                  bool has_scale, float scale) {
+  __shared__ float shared[1024 / kWave];
+  if (*n_routed != 0) return;
+  const int64_t n_slots = n_tokens * top_k;
+  const float wsum = weights_total(weight, wdtype, n_slots, shared);
+  const int64_t n = n_tokens * hidden;
+  float dot = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+    float g = to_float(go[i]);
+    if (has_scale) g = round_through<T>(g * scale);
+    dot += g * to_float(x[i]);
+    if (gx) gx[i] = from_float<T>(g * wsum);
+  }
+  const float total = block_sum_1024(dot, shared);
+  if (gw)
+    for (int64_t s = threadIdx.x; s < n_slots; s += blockDim.x) store_weight_any(gw, wdtype, s, total);
+}
+
 // ---------------------------------------------------------------- index check
 template <bool I64>
 __global__ void claim_rows_kernel(const void* __restrict__ pos, int64_t n_slots, int64_t n_rows,
@@ -776,6 +855,75 @@ int stm_row_parts_to_slots(const float* parts, int n_parts, const int32_t* pos, 
     case STM_F32: row_parts_to_slots_kernel<<<grid, 256, 0, s>>>(parts, n_parts, pos, n_slots, n_rows, static_cast<float*>(out)); break;
     case STM_F16: row_parts_to_slots_kernel<<<grid, 256, 0, s>>>(parts, n_parts, pos, n_slots, n_rows, static_cast<f16_t*>(out)); break;
     case STM_BF16: row_parts_to_slots_kernel<<<grid, 256, 0, s>>>(parts, n_parts, pos, n_slots, n_rows, static_cast<bf16_t*>(out)); break;
+    default: return STM_ERR_UNSUPPORTED;
+  }
+  return launch_status();
+}
+
+int stm_nothing_routed_fwd(const int32_t* n_routed, const void* x, const void* weight, int weight_dtype, void* out,
+                           int64_t n_tokens, int top_k, int64_t hidden, int dtype, int has_scale, float scale,
+                           const void* addend_or_null, stm_stream_t stream) {
+  using namespace stm;
+  if (bad_rows(n_tokens, top_k, hidden)) return STM_ERR_ARG;
+  if (weight_dtype < STM_F32 || weight_dtype > STM_BF16) return STM_ERR_UNSUPPORTED;
+  if (n_tokens == 0 || hidden == 0) return STM_OK;
+  if (!n_routed || !x || !out || (top_k > 0 && !weight)) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  const int64_t n = n_tokens * hidden;
+  const unsigned grid = unsigned(n / 8192 + 1 < 1024 ? n / 8192 + 1 : 1024);
+  const bool hs = has_scale != 0;
+#define STM_LAUNCH(T)                                                                                              \
+  nothing_routed_fwd_kernel<T><<<grid, 1024, 0, s>>>(n_routed, static_cast<const T*>(x), weight, weight_dtype,     \
+                                                     static_cast<T*>(out), n_tokens, top_k, hidden, hs, scale,     \
+                                                     static_cast<const T*>(addend_or_null))
+  switch (dtype) {
+    case STM_F32: STM_LAUNCH(float); break;
+    case STM_F16: STM_LAUNCH(f16_t); break;
+    case STM_BF16: STM_LAUNCH(bf16_t); break;
+    default: return STM_ERR_UNSUPPORTED;
+  }
+#undef STM_LAUNCH
+  return launch_status();
+}
+
+int stm_nothing_routed_bwd(const int32_t* n_routed, const void* grad_out, const void* x, const void* weight,
+                           int weight_dtype, void* grad_x_or_null, void* grad_weight_or_null, int64_t n_tokens,
+                           int top_k, int64_t hidden, int dtype, int has_scale, float scale, stm_stream_t stream) {
+  using namespace stm;
+  if (bad_rows(n_tokens, top_k, hidden)) return STM_ERR_ARG;
+  if (weight_dtype < STM_F32 || weight_dtype > STM_BF16) return STM_ERR_UNSUPPORTED;
+  if (n_tokens == 0 || hidden == 0) return STM_OK;
+  if (!n_routed || !grad_out || !x || (top_k > 0 && !weight)) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  const bool hs = has_scale != 0;
+#define STM_LAUNCH(T)                                                                                            \
+  nothing_routed_bwd_kernel<T><<<1, 1024, 0, s>>>(n_routed, static_cast<const T*>(grad_out),                     \
+                                                  static_cast<const T*>(x), weight, weight_dtype,                \
+                                                  static_cast<T*>(grad_x_or_null), grad_weight_or_null, n_tokens, \
+                                                  top_k, hidden, hs, scale)
+  switch (dtype) {
+    case STM_F32: STM_LAUNCH(float); break;
+    case STM_F16: STM_LAUNCH(f16_t); break;
+    case STM_BF16: STM_LAUNCH(bf16_t); break;
+    default: return STM_ERR_UNSUPPORTED;
+  }
+#undef STM_LAUNCH
+  return launch_status();
+}
+
+int stm_row_dot(const void* a, const void* b, float* out, int64_t n_rows, int64_t hidden, int dtype,
+                stm_stream_t stream) {
+  using namespace stm;
+  if (n_rows < 0 || hidden < 0) return STM_ERR_ARG;
+  if (n_rows == 0) return STM_OK;
+  if (!out || (hidden > 0 && (!a || !b))) return STM_ERR_ARG;
+  hipStream_t s = as_stream(stream);
+  const int rows_per_block = kRowThreads / kWave;
+  const unsigned grid = unsigned((n_rows + rows_per_block - 1) / rows_per_block);
+  switch (dtype) {
+    case STM_F32: row_dot_kernel<<<grid, kRowThreads, 0, s>>>(static_cast<const float*>(a), static_cast<const float*>(b), out, n_rows, hidden); break;
+    case STM_F16: row_dot_kernel<<<grid, kRowThreads, 0, s>>>(static_cast<const f16_t*>(a), static_cast<const f16_t*>(b), out, n_rows, hidden); break;
+    case STM_BF16: row_dot_kernel<<<grid, kRowThreads, 0, s>>>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(b), out, n_rows, hidden); break;
     default: return STM_ERR_UNSUPPORTED;
   }
   return launch_status();

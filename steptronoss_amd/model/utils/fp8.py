@@ -69,10 +69,12 @@ def grouped_gemm_fp8_pow2(a_codes, a_scales, b_codes, b_scales, batch_sizes, out
         offsets = _group_offsets(batch_sizes, dev)
         out = torch.zeros((m_cap, n), device=dev, dtype=out_dtype)
         ws = _gemm_workspace(m_cap, n_groups, dev)
+        # (normalised copies are bound to names: they must outlive the launch)
+        a_c, a_s = a_codes.contiguous(), a_scales.contiguous().float()
+        b_c, b_s = b_codes.contiguous(), b_scales.contiguous().float()
         ok = _lib.try_call(
-            "stm_grouped_gemm_fp8_pow2", ptr(a_codes.contiguous()), ptr(a_scales.contiguous().float()),
-            ptr(b_codes.contiguous()), ptr(b_scales.contiguous().float()), ptr(out), ptr(offsets), n_groups, m_cap, n, k,
-            dtype_code(out_dtype), ptr(ws), ws.numel(), stream(),
+            "stm_grouped_gemm_fp8_pow2", ptr(a_c), ptr(a_s), ptr(b_c), ptr(b_s), ptr(out), ptr(offsets), n_groups, m_cap,
+            n, k, dtype_code(out_dtype), ptr(ws), ws.numel(), stream(),
         )  # fmt: skip
     if not ok:
         raise NotImplementedError("grouped_gemm_fp8_pow2: shape or output type outside the persistent kernel")
@@ -99,9 +101,10 @@ def grouped_gemm_fp8(a_codes, a_scales, b_codes, b_scales, batch_sizes, out_dtyp
         offsets = _group_offsets(batch_sizes, dev)
         out = torch.zeros((m_cap, n), device=dev, dtype=out_dtype)
         ws = _gemm_workspace(m_cap, n_groups, dev)
+        a_c, a_s = a_codes.contiguous(), a_scales.contiguous().float()
+        b_c, b_s = b_codes.contiguous(), b_scales.contiguous().float()
         call(
-            "stm_grouped_gemm_fp8", ptr(a_codes.contiguous()), ptr(a_scales.contiguous().float()),
-            ptr(b_codes.contiguous()), ptr(b_scales.contiguous().float()), ptr(out), ptr(offsets), n_groups, m_cap, n, k,
+            "stm_grouped_gemm_fp8", ptr(a_c), ptr(a_s), ptr(b_c), ptr(b_s), ptr(out), ptr(offsets), n_groups, m_cap, n, k,
             dtype_code(out_dtype), ptr(ws), ws.numel(), stream(),
         )  # fmt: skip
     return out

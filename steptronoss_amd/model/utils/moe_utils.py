@@ -22,6 +22,9 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 
+import collections
+import logging
+
 import torch
 
 from steptronoss_amd import _lib
@@ -29,6 +32,7 @@ from steptronoss_amd._lib import call, try_call, dtype_code, is_i64, ptr, requir
 from steptronoss_amd.utils.optimizable import optimizable
 
 BACKEND_NAME = "hip_gfx950"
+_log = logging.getLogger("steptronoss_amd.moe_utils")
 
 
 @dataclass
@@ -38,9 +42,10 @@ class Settings:
     validate: the stand-alone ``histogram`` / ``index_compute`` read the device status
         words back (one small host sync, as the reference's own checks do) and raise the
         reference's errors.  ``routed_grouped_ffn`` never synchronises unless
-        ``validate_fused`` is set; with it the op also reproduces the reference's early-out
-        for a batch in which no slot is routed (``x * token_weights.sum()``), which needs the
-        routed count on the host.
+        ``validate_fused`` is set; with it an expert id ``>= E`` raises the reference's
+        ``ValueError`` (without it such a slot is treated as not routed).  The reference's
+        early-out for a batch in which no slot is routed (``x * token_weights.sum()``) is taken on
+        the device in either mode.
     weights_before_gemm2: ``routed_grouped_ffn`` with fp32 ``token_weights`` multiplies each
         routed row by its weight right after the SwiGLU (in the first GEMM's epilogue) instead of
         in the combine: the second GEMM is linear in its rows, so the sum is the same up to
@@ -51,12 +56,21 @@ class Settings:
         optimizer/base_gradient_manager.py:153-155) gets its gradient added straight into that
         buffer by the wgrad kernel; autograd then sees ``None`` for it, so no 16-bit gradient
         is written, re-read and added afterwards.
+    probe_activation: ``routed_grouped_ffn`` fuses the SwiGLU into the GEMMs only for an
+        activation it knows by identity; with this switch a callable that merely behaves like the
+        SwiGLU on a probe tensor is replaced as well (and a warning is logged).
+    deferred_id_check: ``routed_grouped_ffn`` copies the routing status words to pinned host
+        memory without waiting; a later call (or ``check_deferred_status()``) that finds such a
+        copy complete raises the reference's "out-of-range" ``ValueError`` for an expert id
+        ``>= E``, one or more steps late but without a synchronisation on the path.
     """
 
     weights_before_gemm2: bool = True
     validate: bool = True
     validate_fused: bool = False
     fuse_main_grad: bool = False
+    probe_activation: bool = False
+    deferred_id_check: bool = True
 
 
 settings = Settings()
@@ -144,6 +158,36 @@ def hip_index_compute(indices: torch.Tensor, expert_histogram: torch.Tensor) -> 
             assert not st[_lib.ST_HIST_NEGATIVE], "expert_histogram must be non-negative"
             assert not st[_lib.ST_HIST_MISMATCH], "expert_histogram does not match number of valid indices"
     return out
+
+
+_PENDING_STATUS: collections.deque = collections.deque()
+
+
+def _defer_status_check(status: torch.Tensor) -> None:
+    """Start an asynchronous copy of the status words to pinned host memory; nothing waits."""
+    host = torch.empty(status.shape, dtype=status.dtype, pin_memory=True)
+    host.copy_(status, non_blocking=True)
+    done = torch.cuda.Event()
+    done.record()
+    _PENDING_STATUS.append((done, host))
+
+
+def check_deferred_status(wait: bool = False) -> None:
+    """Look at the status words of earlier ``routed_grouped_ffn`` calls whose copies have arrived
+    (all of them when ``wait``) and raise the reference's ``ValueError`` (moe_utils.py:119-125) when
+    one of them saw an expert id ``>= E``."""
+    bad = False
+    while _PENDING_STATUS:
+        done, host = _PENDING_STATUS[0]
+        if wait:
+            done.synchronize()
+        elif not done.query():
+            break
+        _PENDING_STATUS.popleft()
+        bad = bad or bool(host[_lib.ST_ID_OUT_OF_RANGE])
+    if bad:
+        _PENDING_STATUS.clear()
+        raise ValueError("top_k_rank contains out-of-range expert index")
 
 
 def route_plan(token_expert_ids: torch.Tensor, n_experts: int):
@@ -501,22 +545,51 @@ class _PermuteKnownRows(torch.autograd.Function):
             return _permute_rows_bwd(grad_out.contiguous(), pos, ctx.hidden), None, None
 
 
+def _nothing_routed_fwd(n_routed, x, weight, out, scale=None, addend=None):
+    """The reference's early-out (moe_utils.py:230-232) without a read-back: a kernel that
+    overwrites ``out`` with ``x * weight.sum()`` (and the optional tail) when the device word
+    ``n_routed`` is zero and does nothing otherwise."""
+    T, K = weight.shape
+    call(
+        "stm_nothing_routed_fwd", ptr(n_routed), ptr(x), ptr(weight), dtype_code(weight.dtype), ptr(out), T, K,
+        x.shape[1], dtype_code(x.dtype), int(scale is not None), float(scale or 0.0), ptr(addend), stream(),
+    )  # fmt: skip
+
+
+def _nothing_routed_bwd(n_routed, grad_out, x, weight, grad_x, grad_weight, scale=None):
+    """Backward of the early-out: overwrites ``grad_x`` / ``grad_weight`` (either may be ``None``)
+    when ``n_routed`` is zero."""
+    T, K = weight.shape
+    call(
+        "stm_nothing_routed_bwd", ptr(n_routed), ptr(grad_out), ptr(x), ptr(weight), dtype_code(weight.dtype),
+        ptr(grad_x), ptr(grad_weight), T, K, x.shape[1], dtype_code(x.dtype), int(scale is not None),
+        float(scale or 0.0), stream(),
+    )  # fmt: skip
+
+
 class _CombineInjective(torch.autograd.Function):
-    """Weighted combine whose position map is known to be injective (index_compute output)."""
+    """Weighted combine whose position map is known to be injective (index_compute output), with
+    the early-out of ``routed_grouped_ffn`` for a batch without a routed slot (``n_routed`` is the
+    device-side count): then the result is ``x * weight.sum()``."""
 
     @staticmethod
-    def forward(ctx, rows, pos, weight):
-        ctx.save_for_backward(rows, pos, weight)
+    def forward(ctx, rows, pos, weight, x, n_routed):
+        ctx.save_for_backward(rows, pos, weight, x, n_routed)
         with torch.cuda.device(rows.device):
-            return _combine_rows(rows, pos, weight)
+            out = _combine_rows(rows, pos, weight)
+            _nothing_routed_fwd(n_routed, x, weight, out)
+        return out
 
     @staticmethod
     def backward(ctx, grad_out):
-        rows, pos, weight = ctx.saved_tensors
+        rows, pos, weight, x, n_routed = ctx.saved_tensors
         with torch.cuda.device(rows.device):
+            go = grad_out.contiguous()
             grad_rows = torch.zeros_like(rows)
-            gw = _combine_rows_bwd(grad_out.contiguous(), rows, pos, weight, grad_rows, None)
-        return grad_rows, None, gw
+            gw = _combine_rows_bwd(go, rows, pos, weight, grad_rows, None)
+            gx = torch.zeros_like(x) if ctx.needs_input_grad[3] else None
+            _nothing_routed_bwd(n_routed, go, x, weight, gx, gw)
+        return grad_rows, None, gw, gx, None
 
 
 def _gemm_swiglu_rows(a: torch.Tensor, w1: torch.Tensor, offsets: torch.Tensor, swiglu_limit, row_scale=None):
@@ -606,8 +679,11 @@ class _FusedRoutedFFN(torch.autograd.Function):
         n_rows = T * K
         with torch.cuda.device(dev):
             _hist, offsets, pos, status = route_plan(token_expert_ids, E)
-            if settings.validate_fused and int(status[_lib.ST_ID_OUT_OF_RANGE]):
-                raise ValueError("top_k_rank contains out-of-range expert index")
+            if settings.validate_fused:
+                if int(status[_lib.ST_ID_OUT_OF_RANGE]):
+                    raise ValueError("top_k_rank contains out-of-range expert index")
+            elif settings.deferred_id_check:
+                _defer_status_check(status)
             live = offsets[E:]  # device word: number of used rows
             xp = torch.empty((n_rows, H), device=dev, dtype=x.dtype)
             call(
@@ -629,10 +705,11 @@ class _FusedRoutedFFN(torch.autograd.Function):
             addend = None if out_addend is None else out_addend.contiguous()
             if w_row is None:
                 out = _combine_rows(y, pos, token_weights, out_scale, addend)
-                ctx.save_for_backward(w1, w2, xp, gu, h, y, pos, offsets, token_weights)
+                ctx.save_for_backward(w1, w2, x, xp, gu, h, y, pos, offsets, token_weights)
             else:  # h and y carry the weights already
                 out = _combine_rows(y, pos, _unit_weights(pos.shape, dev), out_scale, addend)
-                ctx.save_for_backward(w1, w2, xp, gu, h, w_row, pos, offsets, token_weights)
+                ctx.save_for_backward(w1, w2, x, xp, gu, h, w_row, pos, offsets, token_weights)
+            _nothing_routed_fwd(live, x, token_weights, out, out_scale, addend)
         ctx.weighted_rows = w_row is not None
         ctx.limit = swiglu_limit
         ctx.out_scale = out_scale
@@ -643,14 +720,14 @@ class _FusedRoutedFFN(torch.autograd.Function):
     def backward(ctx, grad_out):
         from steptronoss_amd.model.common.feed_forward import swiglu_bwd_rows, swiglu_fwd_rows
 
-        w1, w2, xp, gu, h, y_or_w_row, pos, offsets, token_weights = ctx.saved_tensors
+        w1, w2, x, xp, gu, h, y_or_w_row, pos, offsets, token_weights = ctx.saved_tensors
         T, H, K, E = ctx.shape
         dev = grad_out.device
         need_w1, need_w2, need_x, _, need_tw, _, _, need_addend = ctx.needs_input_grad
         gw1 = gw2 = gx = gtw = None
         with torch.cuda.device(dev):
             live = offsets[E:]
-            go = grad_out.contiguous()
+            go = go_unscaled = grad_out.contiguous()
             dgu = None
             if ctx.weighted_rows:
                 w_row = y_or_w_row
@@ -694,19 +771,35 @@ class _FusedRoutedFFN(torch.autograd.Function):
                 if need_x:
                     dxp = _gemm_rows(dgu, w1, offsets, H, False)
                     gx = _permute_rows_bwd(dxp, pos, H)
+            if need_x or need_tw:  # no routed slot at all: the gradients of x * token_weights.sum()
+                if need_tw and gtw is None:
+                    gtw = torch.zeros_like(token_weights)
+                _nothing_routed_bwd(live, go_unscaled, x, token_weights, gx, gtw if need_tw else None, ctx.out_scale)
         return gw1, gw2, gx, None, (gtw if need_tw else None), None, None, (grad_out if need_addend else None)
 
 
 _ACT_CACHE: dict = {}
+_REFERENCE_SWIGLU = ("steptronoss.model.common.feed_forward", "FeedForwardConfig.activation")
+
+
+def _is_known_swiglu(func) -> bool:
+    """Identity, not behaviour: this package's ``swiglu`` or the reference's own
+    ``FeedForwardConfig.activation`` (feed_forward.py:20-26; a bound method there)."""
+    if getattr(func, "is_steptron_swiglu", False):
+        return True
+    inner = getattr(func, "__func__", func)
+    return (getattr(inner, "__module__", None), getattr(inner, "__qualname__", None)) == _REFERENCE_SWIGLU
 
 
 def _swiglu_limit_of(act, ffn2: int, dtype, device):
     """Decide whether ``act`` is the SwiGLU (optionally clamped) and with which limit.
 
-    Returns ``(True, limit)`` or ``(False, None)``.  A callable is accepted when it is this
-    package's ``swiglu`` (possibly wrapped in ``functools.partial``), or when it reproduces
-    the SwiGLU on a probe tensor whose magnitudes expose a clamp; the verdict is cached per
-    callable.  Anything else is called as-is between two un-fused GEMMs.
+    Returns ``(True, limit)`` or ``(False, None)``.  A callable is accepted when it *is* a known
+    SwiGLU (this package's ``swiglu`` or the reference's ``FeedForwardConfig.activation``,
+    possibly wrapped in a ``functools.partial`` that only binds ``swiglu_limit``).  Anything
+    else is called as-is between two un-fused GEMMs, unless ``settings.probe_activation`` is on:
+    then a callable that reproduces the SwiGLU on a probe tensor whose magnitudes expose a clamp
+    is replaced too, with a log line saying so; the verdict is cached per callable.
     """
     import functools
 
@@ -718,8 +811,10 @@ def _swiglu_limit_of(act, ffn2: int, dtype, device):
     limit = kwargs.pop("swiglu_limit", None)
     if kwargs:
         return False, None
-    if getattr(func, "is_steptron_swiglu", False):
+    if _is_known_swiglu(func):
         return True, limit
+    if not settings.probe_activation:
+        return False, None
     key = (id(func), limit, ffn2, dtype)
     hit = _ACT_CACHE.get(key)
     if hit is not None and hit[0] is func:
@@ -739,6 +834,11 @@ def _swiglu_limit_of(act, ffn2: int, dtype, device):
                 ok = bool((err <= tol).all())
     except Exception:
         ok = False
+    if ok:
+        _log.warning(
+            "routed_grouped_ffn: activation %r behaves like the SwiGLU on a probe and is replaced by the fused "
+            "kernels (settings.probe_activation is on)", func,
+        )  # fmt: skip
     _ACT_CACHE[key] = (func, ok)
     return ok, (limit if ok else None)
 
@@ -777,21 +877,26 @@ def hip_routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights, *, o
                 out = out * out_scale
             return out if out_addend is None else out + out_addend
 
-        if settings.validate_fused and not bool((ids >= 0).any()):
-            # The reference reads the routed count back on the host and, when it is zero, returns
-            # x * sum(weights) (moe_utils.py:230-232).  Only the validating mode pays for that
-            # read-back; without it an all-unrouted batch gives zeros (nothing to combine).
-            return tail(x * token_weights.sum())
+        # (the reference reads the routed count back on the host and, when it is zero, returns
+        # x * sum(weights), moe_utils.py:230-232; here a kernel behind the combine takes that
+        # decision from the device-side count, so there is no read-back)
+        if settings.deferred_id_check:
+            check_deferred_status()
         fused, limit = _swiglu_limit_of(act, w1.shape[1], x.dtype, dev)
         if fused:
             return _FusedRoutedFFN.apply(w1c, w2c, xc, ids, tw, limit, out_scale, out_addend)
-        _hist, offsets, pos, _status = route_plan(ids, E)
+        _hist, offsets, pos, status = route_plan(ids, E)
+        if settings.validate_fused:
+            if int(status[_lib.ST_ID_OUT_OF_RANGE]):
+                raise ValueError("top_k_rank contains out-of-range expert index")
+        elif settings.deferred_id_check:
+            _defer_status_check(status)
         n_rows = T * K
         rows = _no_sync_permute(xc, pos, n_rows)
         rows = _GroupedGemm.apply(rows, w1c, offsets, n_rows, True)
         rows = act(rows)
         rows = _GroupedGemm.apply(rows.contiguous(), w2c, offsets, n_rows, True)
-        return tail(_CombineInjective.apply(rows, pos, tw))
+        return tail(_CombineInjective.apply(rows, pos, tw, xc, offsets[E:]))
 
 
 @optimizable(alternatives={BACKEND_NAME: hip_routed_grouped_ffn, "fused": hip_routed_grouped_ffn})

@@ -6,8 +6,10 @@ row-gather and sorted-segment-sum kernels, the orderings come from its stable so
 supplies device memory and a little index arithmetic on the (small) id vectors.  Like the
 reference, functions whose output length depends on the data read one count back to the host.
 
-Differentiable in ``inp`` (the permutation and its transpose are each other's backward);
-probabilities are treated as constants.
+Differentiable in ``inp`` (the permutation and its transpose are each other's backward) and,
+like the reference, in the probabilities: ``merging_probs`` of ``moe_unpermute`` receives the
+row dot products, ``probs`` of the ``*_with_probs`` functions the scatter-add of the permuted
+probabilities' gradient.
 """
 
 from __future__ import annotations
@@ -86,15 +88,25 @@ class _GatherRows(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, idx):
         ctx.save_for_backward(idx)
-        ctx.n_src = x.shape[0]
+        ctx.src_shape = tuple(x.shape)
         with torch.cuda.device(x.device):
             return _gather_rows_raw(x, idx)
 
     @staticmethod
     def backward(ctx, grad_out):
         (idx,) = ctx.saved_tensors
+        n_src = ctx.src_shape[0]
         with torch.cuda.device(grad_out.device):
-            return _scatter_add_rows_raw(grad_out.contiguous(), idx, ctx.n_src), None
+            g = grad_out.contiguous().reshape(idx.numel(), -1)
+            return _scatter_add_rows_raw(g, idx, n_src).reshape(ctx.src_shape), None
+
+
+def _row_dot(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """``out[j] = <a[j], b[j]>`` in fp32."""
+    a, b = a.contiguous(), b.contiguous()
+    out = torch.empty((a.shape[0],), device=a.device, dtype=torch.float32)
+    call("stm_row_dot", ptr(a), ptr(b), ptr(out), a.shape[0], a.shape[1], dtype_code(a.dtype), stream())
+    return out
 
 
 class _ScatterAddRows(torch.autograd.Function):
@@ -102,18 +114,21 @@ class _ScatterAddRows(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, rows, dest, weight, n_out):
-        ctx.save_for_backward(dest, weight)
+        ctx.save_for_backward(dest, weight, rows if weight is not None else None)
         with torch.cuda.device(rows.device):
             return _scatter_add_rows_raw(rows, dest, n_out, weight)
 
     @staticmethod
     def backward(ctx, grad_out):
-        dest, weight = ctx.saved_tensors
+        dest, weight, rows = ctx.saved_tensors
+        grad_weight = None
         with torch.cuda.device(grad_out.device):
-            g = _gather_rows_raw(grad_out.contiguous(), dest)
+            g = _gather_rows_raw(grad_out.contiguous(), dest)  # zero rows where dest < 0
             if weight is not None:
+                if ctx.needs_input_grad[2]:  # d weight[j] = <d out[dest[j]], rows[j]>
+                    grad_weight = _row_dot(g, rows).to(weight.dtype)
                 g = g * weight.to(g.dtype).unsqueeze(-1)
-        return g, None, None, None
+        return g, None, grad_weight, None
 
 
 def _float_rows_supported(t: torch.Tensor) -> None:
@@ -165,7 +180,7 @@ def _permute_mask_map(inp, routing_map, num_out_tokens, probs):
             if probs.shape != routing_map.shape:
                 raise ValueError("probs must have shape [num_tokens, num_experts]")
             probs_flat = probs.T.contiguous().reshape(-1, 1)
-            permuted_probs = _gather_rows_raw(probs_flat, row_id_map).reshape(-1)
+            permuted_probs = _GatherRows.apply(probs_flat, row_id_map).reshape(-1)
     return output, row_id_map, permuted_probs
 
 
@@ -243,7 +258,7 @@ def moe_unpermute(inp, row_id_map, merging_probs=None, restore_shape=None, map_t
             probs_flat = None if merging_probs is None else merging_probs.reshape(-1, 1)
         weights = None
         if probs_flat is not None:
-            weights = _gather_rows_raw(probs_flat.contiguous(), row_id_map).reshape(-1)
+            weights = _GatherRows.apply(probs_flat.contiguous(), row_id_map).reshape(-1)
         hidden = inp.size(1)
         out_rows = restore_shape[0] if restore_shape is not None else num_tokens
         output = _ScatterAddRows.apply(inp, token_ids, weights, out_rows)
@@ -284,6 +299,4 @@ def moe_sort_chunks_by_index_with_probs(inp, probs, split_sizes, sorted_index):
         raise ValueError("probs and inp must have the same leading dimension")
     require_gpu(inp, probs)
     rows = _chunk_rows(split_sizes, sorted_index, inp.device)
-    with torch.cuda.device(inp.device):
-        out_probs = _gather_rows_raw(probs, rows)
-    return _GatherRows.apply(inp, rows), out_probs
+    return _GatherRows.apply(inp, rows), _GatherRows.apply(probs, rows)

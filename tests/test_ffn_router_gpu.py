@@ -54,6 +54,18 @@ def _torch_swiglu(x, swiglu_limit=None):
     return left * right
 
 
+class _ReferenceLikeConfig:
+    """Stands in for the reference's FeedForwardConfig (feed_forward.py:9-26): same module and
+    qualified name on the method, which is how the backend knows the activation."""
+
+    def activation(self, x, swiglu_limit=None):
+        return _torch_swiglu(x, swiglu_limit)
+
+
+_ReferenceLikeConfig.activation.__module__ = "steptronoss.model.common.feed_forward"
+_ReferenceLikeConfig.activation.__qualname__ = "FeedForwardConfig.activation"
+
+
 def _ffn_case(T, H, K, E, Fh, dtype, act_kind, inv, tol, seed=0, limit=None, std=1.0):
     gen = torch.Generator().manual_seed(seed)
     x = (torch.randn(T, H, generator=gen) * std).to(dtype)
@@ -73,8 +85,10 @@ def _ffn_case(T, H, K, E, Fh, dtype, act_kind, inv, tol, seed=0, limit=None, std
 
     if act_kind == "own":
         act, ref_act = functools.partial(swiglu, swiglu_limit=limit), oracle_act
-    elif act_kind == "torch":  # recognised by its behaviour on a probe
+    elif act_kind in ("torch", "torch_probed"):  # a SwiGLU the backend does not know by identity
         act, ref_act = functools.partial(_torch_swiglu, swiglu_limit=limit), oracle_act
+    elif act_kind == "reference":  # the reference's own activation: a bound method of its config class
+        act, ref_act = functools.partial(_ReferenceLikeConfig().activation, swiglu_limit=limit), oracle_act
     else:  # an activation that is not the SwiGLU: called between two un-fused GEMMs
         act = ref_act = lambda h: F.gelu(h[..., : h.shape[-1] // 2]) + 0.5 * h[..., h.shape[-1] // 2 :]
 
@@ -93,10 +107,22 @@ def _ffn_case(T, H, K, E, Fh, dtype, act_kind, inv, tol, seed=0, limit=None, std
     assert worst <= tol, errs
 
 
-@pytest.mark.parametrize("act_kind", ["own", "torch", "other"])
+@pytest.mark.parametrize("act_kind", ["own", "torch", "torch_probed", "reference", "other"])
 def test_ffn_reference_gpu_test_shape(act_kind):
     # shape of the reference's fused-path test (tests/test_moe_utils_gpu.py:141-220)
-    _ffn_case(256, 64, 2, 8, 96, torch.bfloat16, act_kind, 0.15, BF16_TOL)
+    from steptronoss_amd.profiling import KernelTimer
+
+    old = M.settings.probe_activation
+    M.settings.probe_activation = act_kind == "torch_probed"
+    try:
+        with KernelTimer() as kt:
+            _ffn_case(256, 64, 2, 8, 96, torch.bfloat16, act_kind, 0.15, BF16_TOL)
+    finally:
+        M.settings.probe_activation = old
+    # one autograd node (the fused op) only for an activation known by identity, or by probe when
+    # that is switched on; everything else is called between two un-fused GEMMs
+    fused = "stm_swiglu_fwd" in kt.summary() or "stm_grouped_gemm_swiglu" in kt.summary()
+    assert fused == (act_kind in ("own", "torch_probed", "reference"))
 
 
 @pytest.mark.parametrize(
@@ -269,7 +295,11 @@ def _assert_ids(ids, ref_ids, ref_scores, K):
     rows = torch.nonzero(~same).reshape(-1)
     got_scores = ref_scores[rows].gather(1, ids[rows])
     assert torch.allclose(got_scores, srt[rows, :K], rtol=1e-6, atol=0)
-    return int((~same).sum())
+    n_excused = int((~same).sum())
+    print(f"router ids: {n_excused} of {ids.shape[0]} tokens excused by a near-tie (<= 8 ulp) in the oracle's scores")
+    # sub-ulp near-ties are rare: more than 1 token in 500 (and more than 2) means a real ordering bug
+    assert n_excused <= max(2, ids.shape[0] // 500), f"{n_excused} tokens excused"
+    return n_excused
 
 
 ROUTER_CASES = [
@@ -305,6 +335,12 @@ def test_router_matches_oracle(T, E, K, sig, norm, bias, ng, tg, logit_kind):
     n_swapped = _assert_ids(ids, ref_ids, choice, K)
     if logit_kind == "bf16_grid" and not bias:
         assert n_swapped == 0
+    # the same selection rule on scores computed by the device's own softmax / sigmoid (a second
+    # exp implementation): again equal up to near-ties
+    dev_scores = (torch.sigmoid(lg.detach()) if sig else torch.softmax(lg.detach(), 1)).cpu()
+    dev_choice = O.group_limited_scores(dev_scores if bb is None else dev_scores + bb, ng, tg)
+    dev_ids = torch.sort(dev_choice, dim=1, descending=True, stable=True).indices[:, :K]
+    _assert_ids(ids, dev_ids, dev_choice, K)
     assert torch.equal(hist.cpu(), O.histogram(ids.cpu(), E))
     if n_swapped == 0:
         assert torch.equal(hist.cpu(), ref_hist)
@@ -365,34 +401,109 @@ def test_layer_matches_oracle_on_reduced_configs(name, T, E, tol):
     errs = {
         "out": rel_l2(out, ref),
         "dx": rel_l2(xg.grad, ref_in[0].grad),
-        "dlogits": rel_l2(lg.grad, ref_in[1].grad) / 5,  # sums of many bf16-rounded dot products
         "dw1": rel_l2(blk.experts.w1.grad, ref_in[2].grad),
         "dw2": rel_l2(blk.experts.w2.grad, ref_in[3].grad),
     }
     worst = max(errs.values())
     assert worst <= tol, errs
+    # d logits = R(d weights) + d aux, R the router's backward, which is linear in d weights.  R
+    # cancels most of d weights (for renormalised weights it removes their mean along K), so an
+    # error of d weights that meets the bar is a larger fraction of what is left.  Checked as its
+    # two factors, each to its own bar: the layer's d weights against the oracle's (tol), and the
+    # device's R applied to the device's own d weights against the oracle's R applied to the same
+    # numbers (1e-4, the router test's bar).
+    _, ref_w, ref_aux, _ = O.forward_router(
+        ref_in[1], cfg["K"], use_sigmoid=cfg["sigmoid"], norm_expert_weight=cfg["norm"], n_group=kw["n_group"],
+        topk_group=kw["topk_group"],
+    )  # fmt: skip
+    lw = logits.to(DEV).requires_grad_(True)
+    ids2, w2_, aux2, _ = blk.route(lw)
+    tw = w2_.detach().clone().requires_grad_(True)
+    out2 = blk.experts(xg.detach(), ids2, tw, out_scale=1.5)
+    out2.backward(go.to(DEV))
+    ref_tw = ref_w.detach().clone().requires_grad_(True)
+    ref_out2 = O.routed_grouped_ffn(ref_in[2].detach(), ref_in[3].detach(), O.swiglu, ref_in[0].detach(), ref_ids, ref_tw) * 1.5
+    ref_out2.backward(go.float())
+    assert rel_l2(tw.grad, ref_tw.grad) <= tol, "d weights"
+    size = 1  # one GPU: the reference divides the aux loss by the parallel size (moe_block.py:410)
+    torch.autograd.backward([w2_, aux2], [tw.grad, torch.full_like(aux2, 0.01 / size)])
+    ref_lin = torch.autograd.grad([ref_w, ref_aux], ref_in[1], [tw.grad.cpu().float(), torch.tensor(0.01 / size)])[0]
+    assert rel_l2(lw.grad, ref_lin) <= 1e-4, "router backward on the device's d weights"
+    assert rel_l2(lg.grad, lw.grad) <= 1e-6, "the layer's d logits are R(d weights) + d aux"
+    print(f"{name}: d logits against the oracle end to end: {rel_l2(lg.grad, ref_in[1].grad):.2e}")
 
 
-def test_nothing_routed_early_out_matches_reference_when_validating():
-    # reference moe_utils.py:230-232: with no routed slot at all the op returns x * sum(weights)
-    from steptronoss_amd.model.common.feed_forward import swiglu
-    from steptronoss_amd.model.utils import moe_utils as M
-
+@pytest.mark.parametrize("dtype,wdtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("act_kind", ["own", "other"])
+@pytest.mark.parametrize("validate", [False, True])
+def test_nothing_routed_early_out_matches_reference(dtype, wdtype, act_kind, validate):
+    # reference moe_utils.py:230-232: with no routed slot at all the op returns x * sum(weights);
+    # decided on the device from the routed count, with and without the validating read-backs
     gen = torch.Generator().manual_seed(3)
-    T, H, E, K, F = 12, 32, 4, 2, 16
-    x = torch.randn(T, H, generator=gen).to(DEV)
-    w1 = torch.randn(E, 2 * F, H, generator=gen).to(DEV)
-    w2 = torch.randn(E, H, F, generator=gen).to(DEV)
-    ids = torch.full((T, K), -1, dtype=torch.int64, device=DEV)
+    T, H, E, K, F_ = 12, 32, 4, 2, 16
+    x = torch.randn(T, H, generator=gen).to(dtype)
+    w1 = torch.randn(E, 2 * F_, H, generator=gen).to(dtype)
+    w2 = torch.randn(E, H, F_, generator=gen).to(dtype)
+    ids = torch.full((T, K), -1, dtype=torch.int64)
+    tw = torch.rand(T, K, generator=gen).to(wdtype)
+    go = torch.randn(T, H, generator=gen).to(dtype)
+    act = swiglu if act_kind == "own" else (lambda h: F.gelu(h[..., : h.shape[-1] // 2]) + 0.5 * h[..., h.shape[-1] // 2 :])
+    xr, twr = x.clone().requires_grad_(True), tw.clone().requires_grad_(True)
+    ref = xr * twr.sum()  # the reference's expression, on the same dtypes
+    ref.backward(go)
+    xg, twg = x.to(DEV).requires_grad_(True), tw.to(DEV).requires_grad_(True)
+    old = M.settings.validate_fused
+    try:
+        M.settings.validate_fused = validate
+        out = M.routed_grouped_ffn(w1.to(DEV), w2.to(DEV), act, xg, ids.to(DEV), twg)
+        out.backward(go.to(DEV))
+    finally:
+        M.settings.validate_fused = old
+    tol = 1e-6 if dtype == torch.float32 else 1e-2
+    assert out.dtype == ref.dtype and rel_l2(out, ref) <= tol
+    assert rel_l2(xg.grad, xr.grad) <= tol
+    assert twg.grad.dtype == wdtype and rel_l2(twg.grad, twr.grad) <= tol
+
+
+def test_nothing_routed_early_out_keeps_the_tail_and_leaves_routed_batches_alone():
+    gen = torch.Generator().manual_seed(4)
+    T, H, E, K, F_ = 64, 128, 4, 2, 64
+    x = torch.randn(T, H, generator=gen).bfloat16().to(DEV)
+    w1 = (torch.randn(E, 2 * F_, H, generator=gen) * 0.1).bfloat16().to(DEV)
+    w2 = (torch.randn(E, H, F_, generator=gen) * 0.1).bfloat16().to(DEV)
     tw = torch.rand(T, K, generator=gen).to(DEV)
+    shared = torch.randn(T, H, generator=gen).bfloat16().to(DEV)
+    none = torch.full((T, K), -1, dtype=torch.int64, device=DEV)
+    out = M.hip_routed_grouped_ffn(w1, w2, swiglu, x, none, tw, out_scale=2.5, out_addend=shared)
+    assert torch.equal(out, (x * tw.sum()) * 2.5 + shared)
+    one = none.clone()
+    one[5, 1] = 2  # a single routed slot: the early-out must not fire
+    out = M.hip_routed_grouped_ffn(w1, w2, swiglu, x, one, tw)
+    assert float(out[5].abs().sum()) > 0 and float(out[:5].abs().sum()) == 0 and float(out[6:].abs().sum()) == 0
+
+
+def test_out_of_range_expert_id_surfaces_late_without_a_sync():
+    gen = torch.Generator().manual_seed(5)
+    T, H, E, K, F_ = 64, 64, 4, 2, 32
+    x = torch.randn(T, H, generator=gen).bfloat16().to(DEV)
+    w1 = (torch.randn(E, 2 * F_, H, generator=gen) * 0.1).bfloat16().to(DEV)
+    w2 = (torch.randn(E, H, F_, generator=gen) * 0.1).bfloat16().to(DEV)
+    tw = torch.rand(T, K, generator=gen).to(DEV)
+    ids = make_topk_ids(T, K, E, gen=gen).to(DEV)
+    M.check_deferred_status(wait=True)
+    M.routed_grouped_ffn(w1, w2, swiglu, x, ids, tw)
+    M.check_deferred_status(wait=True)  # a clean batch raises nothing
+    bad = ids.clone()
+    bad[3, 0] = E  # the reference's histogram raises "out-of-range" at once (moe_utils.py:119-125)
+    M.routed_grouped_ffn(w1, w2, swiglu, x, bad, tw)  # no read-back here ...
+    with pytest.raises(ValueError, match="out-of-range"):
+        M.check_deferred_status(wait=True)  # ... the finding arrives with the status copy
+    M.check_deferred_status(wait=True)
     old = M.settings.validate_fused
     try:
         M.settings.validate_fused = True
-        out = M.routed_grouped_ffn(w1, w2, swiglu, x, ids, tw)
-        assert torch.allclose(out, x * tw.sum())
-        M.settings.validate_fused = False
-        out = M.routed_grouped_ffn(w1, w2, swiglu, x, ids, tw)
-        assert float(out.abs().sum()) == 0.0  # no read-back: nothing to combine
+        with pytest.raises(ValueError, match="out-of-range"):
+            M.routed_grouped_ffn(w1, w2, swiglu, x, bad, tw)
     finally:
         M.settings.validate_fused = old
 

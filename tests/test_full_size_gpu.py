@@ -51,8 +51,9 @@ def test_router_invariants(case):
         groups = ids // (E // cfg["n_group"])
         n_groups_used = torch.zeros(T, cfg["n_group"], device=DEV).scatter_(1, groups, 1.0).sum(1)
         assert int(n_groups_used.max()) <= cfg["topk_group"]
-    if case["name"] == "c3":  # the skewed configuration must really be skewed
-        assert int(hist.max()) > 5 * T * K // E
+    if case["name"] == "c3":  # the skewed configuration: a few experts above 10x the mean load, some with none
+        assert int(hist.max()) > 10 * T * K // E
+        assert int((hist == 0).sum()) >= 1
     aux_ref = (torch.softmax(case["logits"].float(), 1) if not cfg["sigmoid"] else None)
     if aux_ref is not None:
         expect = float((aux_ref.mean(0) * hist.float()).sum() * E)

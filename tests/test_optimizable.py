@@ -3,6 +3,7 @@ steptronoss/utils/optimizable.py:22-103)."""
 
 import pytest
 
+from steptronoss_amd import backend  # (registers this package's own six ops on import)
 from steptronoss_amd.utils import optimizable as opt
 
 
@@ -95,3 +96,63 @@ def test_arguments_are_forwarded_unchanged(registry):
     f = _make("f", {"alt": alt})
     opt.set_optimization(f="alt")
     assert f(1, 2, z=3) == 7 and seen == {"a": (1, 2), "k": {"z": 3}}
+
+
+def test_register_backend_joins_a_registry_keyed_like_the_reference(registry):
+    """The reference's six ops live under ``steptronoss.model.utils.moe_utils.<op>``, each with its
+    own alternatives, absent optional backends registered as ``None``
+    (reference moe_utils.py:3-58, 85-89, 435-442).  register_backend adds ``hip_gfx950`` to exactly
+    those six dicts (the caller's own dict objects), touches nothing else, and set_optimization
+    then dispatches to the inserted callables."""
+    ref_alts = {
+        "histogram": {"triton": None},
+        "index_compute": {"triton": None},
+        "routed_grouped_ffn": {"fused": None},
+        "moe_weighted_gather": {"triton": None},
+        "moe_scatter": {"triton": None},
+        "grouped_gemm": {"nv_grouped_gemm": None, "triton_grouped_gemm": None, "npu_gmm": None, "function_imple": lambda *a, **k: "fi"},
+    }  # fmt: skip
+    wrapped = {}
+    for name, alts in ref_alts.items():
+        def body(*a, _name=name, **k):
+            return ("baseline", _name)
+
+        body.__qualname__ = name
+        body.__module__ = "steptronoss.model.utils.moe_utils"
+        wrapped[name] = opt.optimizable(alts)(body)
+    # an op of the same short name elsewhere, and an unrelated op in the same module: left alone
+    def stray(*a, **k):
+        return "stray"
+
+    stray.__qualname__ = "histogram"
+    stray.__module__ = "steptronoss.data.stats"
+    stray_alts = {}
+    opt.optimizable(stray_alts)(stray)
+    def gate(*a, **k):
+        return "gate"
+
+    gate.__qualname__ = "MoEGateFunction"
+    gate.__module__ = "steptronoss.model.utils.moe_utils"
+    gate_alts = {}
+    opt.optimizable(gate_alts)(gate)
+
+    touched = backend.register_backend(registry)
+    assert sorted(touched) == sorted(f"steptronoss.model.utils.moe_utils.{n}" for n in ref_alts)
+    for name, alts in ref_alts.items():
+        assert alts[backend.BACKEND_NAME] is backend.BACKEND_OPS[name]  # inserted into the caller's dict
+        assert registry[f"steptronoss.model.utils.moe_utils.{name}"]["alternatives"] is alts
+    assert backend.BACKEND_NAME not in stray_alts and backend.BACKEND_NAME not in gate_alts
+    assert ref_alts["grouped_gemm"]["nv_grouped_gemm"] is None  # absent backends stay as they were
+
+    # dispatch through the registry: full keys (the short name "histogram" is ambiguous here)
+    calls = []
+    for name in ref_alts:
+        ref_alts[name][backend.BACKEND_NAME] = lambda *a, _n=name, **k: calls.append(_n) or ("hip", _n)
+    opt.set_optimization(**{f"steptronoss.model.utils.moe_utils.{n}": backend.BACKEND_NAME for n in ref_alts})
+    for name, fn in wrapped.items():
+        assert fn(1, 2) == ("hip", name)
+    assert calls == list(ref_alts)
+    opt.set_optimization(grouped_gemm="function_imple")  # resets the other five to their baselines
+    assert wrapped["grouped_gemm"]() == "fi" and wrapped["moe_scatter"]() == ("baseline", "moe_scatter")
+    with pytest.raises(KeyError):
+        opt.set_optimization(histogram=backend.BACKEND_NAME)  # two registered functions share the short name

@@ -147,3 +147,55 @@ def test_mask_map_matches_oracle(P, pad):
     ref_plain = O.moe_unpermute(ref_out, ref_rid, restore_shape=x.shape)
     plain = P.moe_unpermute(out, rid, restore_shape=x.shape)
     assert rel_l2(plain, ref_plain) <= 1e-6
+
+
+def test_probabilities_receive_gradients_like_the_reference(P):
+    """The reference's helpers are plain differentiable torch code (permute_utils.py:43-89,
+    157-234): merging_probs gets d out . row, probs the scatter-add of d permuted_probs."""
+    gen = torch.Generator().manual_seed(9)
+    T, E, H = 120, 12, 40
+    mask = torch.rand(T, E, generator=gen) < 0.2
+    probs = torch.rand(T, E, generator=gen) * mask
+    x = torch.randn(T, H, generator=gen)
+    go = torch.randn(T, H, generator=gen)
+    gp = torch.randn(int(mask.sum()), generator=gen)
+
+    # mask map: permute_with_probs -> (rows * permuted_probs) -> unpermute with merging_probs
+    xr, pr, mr = x.clone().requires_grad_(True), probs.clone().requires_grad_(True), probs.clone().requires_grad_(True)
+    r_out, r_rid, r_pp = O.moe_permute(xr, mask, probs=pr)
+    r_back = O.moe_unpermute(r_out * r_pp.unsqueeze(1), r_rid, merging_probs=mr, restore_shape=x.shape)
+    (r_back * go).sum().add((r_pp * gp).sum()).backward()
+    xg, pg, mg = (t.clone().to(DEV).requires_grad_(True) for t in (x, probs, probs))
+    out, pp, rid = P.moe_permute_with_probs(xg, pg, mask.to(DEV))
+    back = P.moe_unpermute(out * pp.unsqueeze(1), rid, merging_probs=mg, restore_shape=x.shape)
+    (back * go.to(DEV)).sum().add((pp * gp.to(DEV)).sum()).backward()
+    assert rel_l2(back, r_back) <= 1e-6
+    assert mg.grad is not None and rel_l2(mg.grad, mr.grad) <= 1e-5
+    assert pg.grad is not None and rel_l2(pg.grad, pr.grad) <= 1e-5
+    assert rel_l2(xg.grad, xr.grad) <= 1e-5
+    assert float(mg.grad.cpu()[~mask].abs().sum()) == 0.0  # unrouted entries take no part
+
+    # index map
+    K = 3
+    ids = torch.randint(-2, E, (T, K), generator=gen)
+    w = torch.rand(T, K, generator=gen)
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    r_out, r_rid = O.moe_permute(xr, ids, map_type="index")
+    (O.moe_unpermute(r_out, r_rid, merging_probs=wr, restore_shape=x.shape, map_type="index") * go).sum().backward()
+    xg, wg = x.clone().to(DEV).requires_grad_(True), w.clone().to(DEV).requires_grad_(True)
+    out, rid = P.moe_permute(xg, ids.to(DEV), map_type="index")
+    (P.moe_unpermute(out, rid, merging_probs=wg, restore_shape=x.shape, map_type="index") * go.to(DEV)).sum().backward()
+    assert wg.grad is not None and rel_l2(wg.grad, wr.grad) <= 1e-5
+    assert rel_l2(xg.grad, xr.grad) <= 1e-5
+
+    # chunk sort with probabilities
+    sizes, order = torch.tensor([50, 30, 40]), torch.tensor([2, 0, 1])
+    pv = torch.rand(T, generator=gen)
+    gv = torch.randn(T, generator=gen)
+    pvr = pv.clone().requires_grad_(True)
+    _, r_p = O.moe_sort_chunks_by_index(x, sizes, order, probs=pvr)
+    (r_p * gv).sum().backward()
+    pvg = pv.clone().to(DEV).requires_grad_(True)
+    _, p_dev = P.moe_sort_chunks_by_index_with_probs(x.to(DEV), pvg, sizes, order)
+    (p_dev * gv.to(DEV)).sum().backward()
+    assert rel_l2(pvg.grad, pvr.grad) <= 1e-6
