@@ -37,6 +37,24 @@ inline size_t tile_table_bytes(int64_t m_cap, int n_groups, int bm) {
   return 16 + size_t(max_m_tiles(m_cap, n_groups, bm)) * sizeof(MTile);
 }
 
+// Exact unsigned 32-bit division by a divisor known on the host: a multiply-high, an add and
+// two shifts on the device instead of a division routine.
+struct FastDivider {
+  uint32_t mul = 1, shift1 = 0, shift2 = 0;
+  FastDivider() = default;
+  explicit FastDivider(uint32_t d) {
+    uint32_t l = 0;
+    while ((uint64_t(1) << l) < d) ++l;  // ceil(log2 d)
+    mul = uint32_t(((uint64_t(1) << 32) * ((uint64_t(1) << l) - d)) / d + 1);
+    shift1 = l < 1 ? l : 1;
+    shift2 = l > 0 ? l - 1 : 0;
+  }
+  __host__ __device__ __forceinline__ uint32_t quotient(uint32_t n) const {
+    const uint32_t t = uint32_t((uint64_t(mul) * n) >> 32);  // one multiply-high
+    return (t + ((n - t) >> shift1)) >> shift2;
+  }
+};
+
 // Arguments shared by the MFMA kernels (rows form: n_j = N, n_k = K; wgrad form: n_i = P, n_j = Q).
 struct GemmArgs {
   const void* a;
@@ -49,6 +67,7 @@ struct GemmArgs {
   int64_t b_group, c_group;
   int n_i, n_j, n_k;
   int tiles_i, tiles_j;
+  FastDivider div_i, div_j;  // division of tile ids by tiles_i / tiles_j (persistent kernels)
   int n_groups;
   int64_t blocks_padded;
   // SwiGLU fused into the epilogue (rows form only):

@@ -37,6 +37,7 @@
 //            the four rows a transposing read touches land in the four quarters of the banks.
 // A wave-wide buffer_load ... lds writes 1024 consecutive LDS bytes (lane l at +16*l), so the
 // swizzle is applied on the global-address side.
+#include <cstdlib>
 #include <type_traits>
 
 #include "gemm_common.hpp"
@@ -72,6 +73,7 @@ struct Mfma<f16_t> {
 
 constexpr int kStagesBytesLog2 = 17;  // the stages of a workgroup fill 128 KiB of LDS, whatever their depth
 constexpr int kEpilogueBytes = 32768;  // output staging of all waves, behind the stages
+constexpr int kStoreAux = 2;  // cache policy bits of the output stores: nt (streamed; the outputs are not re-read soon)
 
 template <typename T>
 struct alignas(sizeof(T) * 4) Pack4 {
@@ -84,6 +86,20 @@ struct alignas(sizeof(T) * 8) Pack8 {
 template <typename T>
 __device__ __forceinline__ float round_to(float f) {
   return to_float(from_float<T>(f));
+}
+
+// Tables the scheduler walks (M-tile list, group offsets) are read through the scalar data cache:
+// a uniform address, the "constant" address space, no vector-memory operation.  A vector load
+// here would make the compiler wait for the vector-memory counter to reach zero, i.e. for every
+// load of later stages and every output store still in flight, at each change of tile.
+typedef __attribute__((address_space(4))) const int32_t* const_i32_ptr;
+typedef __attribute__((address_space(4))) const i32x4_t* const_i32x4_ptr;
+__device__ __forceinline__ int32_t scalar_load(const int32_t* p, int64_t index) {
+  return reinterpret_cast<const_i32_ptr>(reinterpret_cast<uintptr_t>(p))[index];
+}
+__device__ __forceinline__ MTile scalar_load(const MTile* p, int64_t index) {
+  const i32x4_t v = reinterpret_cast<const_i32x4_ptr>(reinterpret_cast<uintptr_t>(p))[index];
+  return MTile{v[0], v[1], v[2], v[3]};
 }
 
 // Raw buffer descriptor over [base, base + bytes): reads past the end return zero.
@@ -227,9 +243,17 @@ enum Epilogue { kStore = 0, kSwigluFwd = 1, kSwigluBwd = 2, kAccumF32 = 3, kStor
 //   unchanged; the products run on v_mfma_scale_f32_32x32x64_f8f6f4, which multiplies each
 //   operand by a power of two given as an exponent byte: the per-row, per-block scales go in
 //   there and the fp32 accumulators need no rescaling.  T is the output type.
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int kBK, int EPI>
+// PP (ping-pong; 8 waves, stages of 32): the two waves of a SIMD take turns.  A step of a wave
+// has a memory half (read the MFMA fragments of the stage from LDS, issue this wave's share of
+// the loads of a later stage) and a matrix half (nothing but the MFMAs on those fragments).
+// One wave of a SIMD meets the workgroup barrier of the step between its halves, the other
+// after both, so that between two barriers one multiplies while the other reads and then they
+// swap: the matrix pipe is fed back to back, no MFMA waits for an LDS read of its own wave,
+// and the epilogue of one wave runs under the MFMAs of its partner.
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int kBK, int EPI, bool PP>
 __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs p) {
   static_assert(kBK == 64 || kBK == 32, "contraction elements per stage");
+  static_assert(!PP || (WAVES == 8 && kBK == 32 && EPI != kStoreFp8), "ping-pong: 8 waves, stages of 32");
   static_assert(EPI == kStore || EPI == kAccumF32 || (WAVES == 8 && !WGRAD && !A_KM),
                 "fused SwiGLU epilogues: rows form, 8 waves");
   static_assert(EPI != kAccumF32 || (WAVES == 8 && WGRAD), "accumulation into an fp32 buffer: wgrad, 8 waves");
@@ -265,8 +289,10 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   // its workgroups take them round-robin, so that at any time they sit next to each other.
   // (values loaded from memory are pinned to scalar registers at once: all tile bookkeeping
   // below is wave-uniform and must stay on the scalar unit)
-  const int64_t n_tiles = WGRAD ? int64_t(p.n_groups) * p.tiles_i * p.tiles_j
-                                : int64_t(__builtin_amdgcn_readfirstlane(p.header[0])) * p.tiles_j;
+  // (tile ids fit 31 bits, checked on the host; divisions by the tile-grid extents use the
+  // host-prepared multipliers: a tile change costs a handful of scalar instructions)
+  const int n_tiles = WGRAD ? p.n_groups * p.tiles_i * p.tiles_j
+                            : scalar_load(p.header, 0) * p.tiles_j;
   // Normally an XCD owns a contiguous range of tile ids.  The work of a wgrad tile grows with
   // its expert's row count; when that is very uneven (largest expert above three times the
   // mean) a contiguous range would leave one XCD with all tiles of a large expert, so then the
@@ -280,28 +306,61 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       most = rows > most ? rows : most;
     }
     most = __builtin_amdgcn_readfirstlane(wave_max(most));
-    const int total = __builtin_amdgcn_readfirstlane(p.offsets[p.n_groups]);
+    const int total = scalar_load(p.offsets, p.n_groups);
     dealt = int64_t(most) * p.n_groups > 3 * int64_t(total);
   }
-  const int64_t deal = p.tiles_j;
-  const int64_t per_xcd =
-      dealt ? (n_tiles / deal + kNumXcd - 1) / kNumXcd * deal : (n_tiles + kNumXcd - 1) / kNumXcd;  // upper bound
-  const int64_t xcd = blockIdx.x % kNumXcd;
-  const int64_t wgs_per_xcd = gridDim.x / kNumXcd;
-  auto tile_id = [&](int64_t k) -> int64_t {
+  const int deal = p.tiles_j;
+  const int per_xcd = dealt ? (int(p.div_j.quotient(uint32_t(n_tiles))) + kNumXcd - 1) / kNumXcd * deal
+                            : (n_tiles + kNumXcd - 1) / kNumXcd;  // upper bound
+  const int xcd = blockIdx.x % kNumXcd;
+  const int wgs_per_xcd = gridDim.x / kNumXcd;
+  auto tile_id = [&](int k) -> int {
     if (k >= per_xcd) return -1;
-    const int64_t id = dealt ? ((k / deal) * kNumXcd + xcd) * deal + k % deal : xcd * per_xcd + k;
+    int id = xcd * per_xcd + k;
+    if (dealt) {
+      const int row = int(p.div_j.quotient(uint32_t(k)));
+      id = (row * kNumXcd + xcd) * deal + (k - row * deal);
+    }
     return id < n_tiles ? id : -1;
   };
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int hw_wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int lane = threadIdx.x % kWave;
+  // The role of a wave (which part of the tile it computes, which loads it issues) is numbered by
+  // `wave`.  Ping-pong pairs the two waves that share a SIMD: they get roles 2s and 2s + 1 (s =
+  // 0..3) and the role's low bit is the group that decides who starts with the memory half step.
+  // Which waves share a SIMD is read from the hardware id register; should the eight waves ever
+  // not sit two per SIMD the plain numbering is kept (correct, only slower).
+  int role = hw_wave;
+  if constexpr (PP) {
+    int* simd_of = reinterpret_cast<int*>(smem + (size_t(1) << kStagesBytesLog2));
+    const int simd = __builtin_amdgcn_s_getreg((1 << 11) | (4 << 6) | 4);  // HW_ID bits 5:4 = SIMD_ID
+    if (lane == 0) simd_of[hw_wave] = simd;
+    __syncthreads();
+    int pair_slot[4] = {0, 0, 0, 0};  // waves seen so far per SIMD
+    bool two_each = true;
+    int mine = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const int sw = __builtin_amdgcn_readfirstlane(simd_of[w]) & 3;
+      int rank = 0;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (sw == q) rank = pair_slot[q]++;
+      if (w == hw_wave) mine = sw * 2 + rank;
+      two_each = two_each && rank < 2;
+    }
+    __syncthreads();
+    role = two_each ? mine : hw_wave;
+  }
+  const int wave = __builtin_amdgcn_readfirstlane(role);
   // rows of B a wave loads per stage start at tile row wave * (BN / WAVES)
   const uint32_t b_rows_per_wave = BN / WAVES;
-  auto locate = [&](int64_t id, TileState<T>& t) {
+  auto locate = [&](int id, TileState<T>& t) {
     const T* a = static_cast<const T*>(p.a);
     const T* b = static_cast<const T*>(p.b);
     T* c = static_cast<T*>(p.c);
-    const int jt = int(id % p.tiles_j);
+    const int id_over_j = int(p.div_j.quotient(uint32_t(id)));
+    const int jt = id - id_over_j * p.tiles_j;
     const int j0 = EPI == kSwigluFwd ? jt * (BN / 2) : jt * BN;
     int n_k;
     uint32_t a_bytes, b_bytes;
@@ -312,11 +371,10 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     t.c2 = nullptr;
     t.soff_b0 = 0;
     if constexpr (WGRAD) {
-      const int64_t rest = id / p.tiles_j;
-      const int it = int(rest % p.tiles_i);
-      const int64_t g = rest / p.tiles_i;
-      const int64_t lo = __builtin_amdgcn_readfirstlane(p.offsets[g]);
-      const int64_t hi = __builtin_amdgcn_readfirstlane(p.offsets[g + 1]);
+      const int64_t g = int64_t(p.div_i.quotient(uint32_t(id_over_j)));
+      const int it = id_over_j - int(g) * p.tiles_i;
+      const int64_t lo = scalar_load(p.offsets, g);
+      const int64_t hi = scalar_load(p.offsets, g + 1);
       n_k = hi > lo ? int(hi - lo) : 0;
       const int i0 = it * BM;
       t.valid_i = p.n_i - i0;
@@ -332,10 +390,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       a_bytes = ab > 0 ? uint32_t(ab) : 0u;
       b_bytes = bb > 0 ? uint32_t(bb) : 0u;
     } else {
-      MTile mt = p.tiles[id / p.tiles_j];
-      mt.group = __builtin_amdgcn_readfirstlane(mt.group);
-      mt.row0 = __builtin_amdgcn_readfirstlane(mt.row0);
-      mt.rows = __builtin_amdgcn_readfirstlane(mt.rows);
+      const MTile mt = scalar_load(p.tiles, id_over_j);
       n_k = p.n_k;
       t.valid_i = mt.rows;
       t.row0 = mt.row0;
@@ -381,6 +436,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   // specialised on the number of live sub-blocks of the wave.
   const int wave_row = wave / 2;
   const int wave_j = (wave % 2) * (BN / 2);
+  const int group = wave % 2;  // ping-pong: group 0 starts with a memory half step, group 1 a half step later
 
   // ---- the load cursor: walks the stream of stages ahead of the MFMAs.  Its state is
   // wave-uniform (scalar registers).  Moving to the next step of a tile costs a handful of
@@ -396,7 +452,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   uint32_t l_soff_a = l_soff_a0, l_soff_b = l_soff_b0;
   uint32_t l_slot = 0;  // byte offset of the LDS slot being filled
   int l_step = 0, l_n_steps = 1;
-  int64_t l_k = 0;
+  int l_k = 0;
   auto load_tile = [&](const TileState<T>& t) {
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
@@ -426,7 +482,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     l_soff_b += plan_b.step_bytes;
     if (++l_step >= l_n_steps) {
       l_k += wgs_per_xcd;
-      const int64_t id = tile_id(l_k);
+      const int id = tile_id(l_k);
       TileState<T> t;
       if (id >= 0) {
         locate(id, t);
@@ -443,7 +499,9 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   // and the loads of its second stage are partly issued; on exit the same holds for the next
   // tile if there is one (`more`).
   uint32_t c_slot = 0;  // byte offset of the LDS slot the MFMAs read
-  auto run_tile = [&](auto atm_tag, const TileState<T>& cur, bool more, uint4 (&f0a)[TM], uint4 (&f0b)[TN]) {
+  // prev_subs: live sub-blocks this wave had in the tile before (0 for the first tile)
+  auto run_tile = [&](auto atm_tag, const TileState<T>& cur, bool more, uint4 (&f0a)[TM], uint4 (&f0b)[TN],
+                      int prev_subs) {
     constexpr int ATM = decltype(atm_tag)::value;
     constexpr int AR = ATM > 0 ? ATM : 1;
     // The lane index as seen by this tile's address arithmetic: passed through an opaque asm so
@@ -459,10 +517,12 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     uint4 fa[2][TM], fb[2][TN];
+    if constexpr (!PP) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) fa[0][i] = f0a[i];
+      for (int i = 0; i < TM; ++i) fa[0][i] = f0a[i];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fb[0][j] = f0b[j];
+      for (int j = 0; j < TN; ++j) fb[0][j] = f0b[j];
+    }
 
     // one 16-wide slice: the MFMAs of register set `set`; in their shadow the LDS reads of
     // slice `kk_next` of stage `stage_next` into the other set (one read per two MFMAs) and
@@ -500,7 +560,74 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     using CL = std::integral_constant<int, kLoads>;
 
     const int n_steps = cur.n_steps;
-    if constexpr (kFp8) {
+    if constexpr (PP) {
+      static_assert(kBK == 32 && kStages >= 3, "two 16-wide slices per stage, loads at least two stages ahead");
+      // The counter of outstanding vector-memory operations retires in order, stores included.
+      // The stores of the previous tile's epilogue sit between the loads issued before and after
+      // it; while the loads waited for are older than those stores, the stores may stay in
+      // flight (they get the first kStages - 2 steps of a tile to complete).
+      // (vector-memory operations a wave's epilogue issues per live 32-row sub-block, at least)
+      constexpr int kOpsPerSub = EPI == kStore ? kColRounds * 4 : EPI == kSwigluFwd ? 12 : EPI == kSwigluBwd ? 36 : TN * 8;
+      constexpr int kRelaxed1 = kInFlight + kOpsPerSub < 63 ? kInFlight + kOpsPerSub : 63;
+      constexpr int kRelaxed2 = kInFlight + 2 * kOpsPerSub < 63 ? kInFlight + 2 * kOpsPerSub : 63;
+      auto wait_for_loads = [&](int step) {
+        if (step < kStages - 2 && prev_subs == 2)
+          asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kRelaxed2) : "memory");
+        else if (step < kStages - 2 && prev_subs == 1)
+          asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kRelaxed1) : "memory");
+        else
+          asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kInFlight) : "memory");
+      };
+      for (int step = 0; step < n_steps; ++step) {
+        // ---- memory half step: the fragments of this stage, then this wave's loads of the stage
+        // kStages - 1 ahead (into the slot both groups finished reading a half step ago)
+        const unsigned char* ta = smem + c_slot;
+        const unsigned char* tb = ta + PlanA::kStageBytes;
+        if constexpr (ATM > 0) {
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+            for (int i = 0; i < ATM; ++i)
+              fa[kk][i] = read_fragment<BM, A_KM, kBK>(ta, (WROWS * i + wave_row) * 32, kk, tl);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[kk][j] = read_fragment<BN, B_KM, kBK>(tb, wave_j + j * 32, kk, tl);
+          }
+        }
+        c_slot = (c_slot + kStageBytes) & (kStages * kStageBytes - 1);
+        issue_loads(C0{}, CL{});
+        advance_loads();
+        // One workgroup barrier per step.  Group 1 meets it between its two halves, group 0 after
+        // both: between two barriers group 0 reads and then multiplies stage s while group 1
+        // multiplies stage s - 1 (read before the barrier) and then reads stage s, so the MFMAs of
+        // one wave of a SIMD run under the LDS reads and load issue of the other.  Before the
+        // barrier a wave makes sure that its loads of the stage read next have landed (all but
+        // those of the kStages - 2 youngest stages) and that its LDS reads of this stage are done
+        // (the slot is refilled after the barrier).
+        if (group == 1) {
+          wait_for_loads(step);
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          __builtin_amdgcn_sched_barrier(0);
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (ATM > 0) {
+          __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int i = 0; i < ATM; ++i)
+#pragma unroll
+              for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(fb[kk][j], fa[kk][i], acc[i][j]);
+          __builtin_amdgcn_s_setprio(0);
+        }
+        if (group == 0) {
+          wait_for_loads(step);
+          __builtin_amdgcn_sched_barrier(0);
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    } else if constexpr (kFp8) {
       // One step = one 128-code scale block = two MFMAs (64 codes each) per pair of sub-blocks.
       // A lane feeds the MFMA 32 codes of its row: the 16-byte chunks 2h and 2h+1 (h = lane / 32)
       // of the 64-byte half row; both operands use the same rule, so matching codes meet.
@@ -606,10 +733,12 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       c_slot = (c_slot + kStageBytes) & (kStages * kStageBytes - 1);
       slice(1, true, c_slot, 0, C0{}, CE{});
     }
+    if constexpr (!PP) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) f0a[i] = fa[0][i];
+      for (int i = 0; i < TM; ++i) f0a[i] = fa[0][i];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) f0b[j] = fb[0][j];
+      for (int j = 0; j < TN; ++j) f0b[j] = fb[0][j];
+    }
 
     // ---- epilogue.  In the accumulators a lane owns row (lane % 32) of a sub-block and, per
     // group of four registers, four consecutive columns starting at (r/4)*8 + (lane/32)*4:
@@ -653,7 +782,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
           const uint4 v = *reinterpret_cast<const uint4*>(buf + row * 256 + ((rd_c16 ^ (row & 15)) * 16));
           __builtin_amdgcn_raw_buffer_store_b128(
               __builtin_bit_cast(u32x4_t, v), rsrc_c,
-              col_live ? uint32_t(row0 + row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset, 0, 0);
+              col_live ? uint32_t(row0 + row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset, 0, kStoreAux);
         }
       }
     } else {
@@ -707,7 +836,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
               const float4 sum = make_float4(old[it].x + v.x, old[it].y + v.y, old[it].z + v.z, old[it].w + v.w);
               __builtin_amdgcn_raw_buffer_store_b128(
                   __builtin_bit_cast(u32x4_t, sum), rsrc_c,
-                  col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes_c + uint32_t(col) * 4u : kDroppedOffset, 0, 0);
+                  col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes_c + uint32_t(col) * 4u : kDroppedOffset, 0, kStoreAux);
             }
           }
         }
@@ -724,8 +853,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
             for (int it = 0; it < 4; ++it)
               __builtin_amdgcn_raw_buffer_store_b128(
                   __builtin_bit_cast(u32x4_t, staged(it)), rsrc_c,
-                  col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset, 0,
-                  0);
+                  col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset, 0, kStoreAux);
           }
         }
       } else {
@@ -756,8 +884,7 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
               for (int it = 0; it < 4; ++it)
                 __builtin_amdgcn_raw_buffer_store_b128(
                     __builtin_bit_cast(u32x4_t, staged(it)), rsrc,
-                    col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes + byte0 + uint32_t(col) * 2u : kDroppedOffset,
-                    0, 0);
+                    col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes + byte0 + uint32_t(col) * 2u : kDroppedOffset, 0, kStoreAux);
             };
             stage([&](int jj, int q, int e) { return acc[i][jj][q * 4 + e]; });
             store_round(rsrc_c, row_bytes_c, 0u);
@@ -834,9 +961,9 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
                   eight(std::false_type{});
                 const uint32_t at =
                     col_live ? uint32_t(row0 + it * 8 + rd_row) * row_bytes_c + uint32_t(col) * 2u : kDroppedOffset;
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, og), rsrc_c, at, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, og), rsrc_c, at, 0, kStoreAux);
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, ou), rsrc_c,
-                                                       col_live ? at + up_bytes : kDroppedOffset, 0, 0);
+                                                       col_live ? at + up_bytes : kDroppedOffset, 0, kStoreAux);
               }
             }
             // the eight lanes of a row (rd_c = 0..7) add up in the last of them, which stores
@@ -857,8 +984,8 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   };
 
   // ---- prologue: first tile, its first stage in full and the head of its second
-  int64_t k = blockIdx.x / kNumXcd;
-  int64_t id = tile_id(k);
+  int k = blockIdx.x / kNumXcd;
+  int id = tile_id(k);
   if (id < 0) return;
   TileState<T> cur;
   locate(id, cur);
@@ -871,39 +998,48 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     issue_loads(std::integral_constant<int, 0>{}, std::integral_constant<int, kLoads>{});
     advance_loads();
   }
-  issue_loads(std::integral_constant<int, 0>{}, std::integral_constant<int, kEarly>{});
-  // stage 0 has landed once at most the younger loads are outstanding
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"((kStages - 2) * kLoads + kEarly) : "memory");
-  __syncthreads();
   uint4 f0a[TM], f0b[TN];
+  if constexpr (PP) {
+    // stage 0 has landed once at most the two younger stages are outstanding
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kInFlight) : "memory");
+    __syncthreads();
+  } else {
+    issue_loads(std::integral_constant<int, 0>{}, std::integral_constant<int, kEarly>{});
+    // stage 0 has landed once at most the younger loads are outstanding
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"((kStages - 2) * kLoads + kEarly) : "memory");
+    __syncthreads();
 #pragma unroll
-  for (int j = 0; j < TN; ++j) f0b[j] = read_fragment<BN, B_KM, kBK>(smem + PlanA::kStageBytes, wave_j + j * 32, 0, lane);
+    for (int j = 0; j < TN; ++j)
+      f0b[j] = read_fragment<BN, B_KM, kBK>(smem + PlanA::kStageBytes, wave_j + j * 32, 0, lane);
 #pragma unroll
-  for (int i = 0; i < TM; ++i) f0a[i] = read_fragment<BM, A_KM, kBK>(smem, (WROWS * i + wave_row) * 32, 0, lane);
+    for (int i = 0; i < TM; ++i) f0a[i] = read_fragment<BM, A_KM, kBK>(smem, (WROWS * i + wave_row) * 32, 0, lane);
+  }
 
+  int prev_subs = 0;
   while (true) {
-    const int64_t next_id = tile_id(k + wgs_per_xcd);
+    const int next_id = tile_id(k + wgs_per_xcd);
     const bool more = next_id >= 0;
     const int live_sub = (cur.valid_i < BM ? cur.valid_i + 31 : BM) / 32;  // live 32-row sub-blocks
     const int my_sub =
         __builtin_amdgcn_readfirstlane((live_sub + WROWS - 1 - wave_row) / WROWS);  // those of this wave row
     if constexpr (TM == 4) {
       switch (my_sub) {
-        case 0: run_tile(std::integral_constant<int, 0>{}, cur, more, f0a, f0b); break;
-        case 1: run_tile(std::integral_constant<int, 1>{}, cur, more, f0a, f0b); break;
-        case 2: run_tile(std::integral_constant<int, 2>{}, cur, more, f0a, f0b); break;
-        case 3: run_tile(std::integral_constant<int, 3>{}, cur, more, f0a, f0b); break;
-        default: run_tile(std::integral_constant<int, 4>{}, cur, more, f0a, f0b); break;
+        case 0: run_tile(std::integral_constant<int, 0>{}, cur, more, f0a, f0b, prev_subs); break;
+        case 1: run_tile(std::integral_constant<int, 1>{}, cur, more, f0a, f0b, prev_subs); break;
+        case 2: run_tile(std::integral_constant<int, 2>{}, cur, more, f0a, f0b, prev_subs); break;
+        case 3: run_tile(std::integral_constant<int, 3>{}, cur, more, f0a, f0b, prev_subs); break;
+        default: run_tile(std::integral_constant<int, 4>{}, cur, more, f0a, f0b, prev_subs); break;
       }
     } else {
       static_assert(TM == 2, "4 or 8 waves");
       switch (my_sub) {
-        case 0: run_tile(std::integral_constant<int, 0>{}, cur, more, f0a, f0b); break;
-        case 1: run_tile(std::integral_constant<int, 1>{}, cur, more, f0a, f0b); break;
-        default: run_tile(std::integral_constant<int, 2>{}, cur, more, f0a, f0b); break;
+        case 0: run_tile(std::integral_constant<int, 0>{}, cur, more, f0a, f0b, prev_subs); break;
+        case 1: run_tile(std::integral_constant<int, 1>{}, cur, more, f0a, f0b, prev_subs); break;
+        default: run_tile(std::integral_constant<int, 2>{}, cur, more, f0a, f0b, prev_subs); break;
       }
     }
     if (!more) break;
+    prev_subs = my_sub;
     k += wgs_per_xcd;
     locate(next_id, cur);
   }
@@ -924,9 +1060,9 @@ int persistent_grid() {
   return cached;
 }
 
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int BK, int EPI>
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int BK, int EPI, bool PP>
 int launch_waves(const GemmArgs& p, hipStream_t s) {
-  auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD, WAVES, BK, EPI>;
+  auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD, WAVES, BK, EPI, PP>;
   constexpr size_t smem = (size_t(1) << kStagesBytesLog2) + size_t(kEpilogueBytes);
   static bool configured = false;
   if (!configured) {
@@ -942,14 +1078,42 @@ int launch_waves(const GemmArgs& p, hipStream_t s) {
 // Two waves per SIMD: measured faster than one (4 waves) on every product of the expert FFN.
 constexpr int kGemmWaves = 8;
 
+// Two schedules of the main loop exist: "interleaved" (every wave mixes its LDS reads and loads
+// into its own MFMAs; stages of 64 when both operands are K-contiguous) and "ping-pong".  Each
+// product runs the one measured faster for it on the expert-FFN shapes: ping-pong for the weight
+// gradients and the fused SwiGLU forward (its epilogue runs under the partner wave's MFMAs),
+// interleaved for the rest.  STM_GEMM_SCHEDULE=interleaved / pingpong forces one for all.
+enum Product { kRowsFwd, kRowsDgrad, kFusedFwd, kFusedBwd, kWgrad };
+bool use_pingpong(Product which) {
+  static const int forced = [] {
+    const char* v = getenv("STM_GEMM_SCHEDULE");
+    return !v ? 0 : v[0] == 'i' ? 1 : v[0] == 'p' ? 2 : 0;
+  }();
+  if (forced) return forced == 2;
+  return which == kWgrad || which == kFusedFwd;
+}
+
 template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int BK, int EPI = kStore>
 int launch(const GemmArgs& p, hipStream_t s) {
-  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, kGemmWaves, BK, EPI>(p, s);
+  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, kGemmWaves, BK, EPI, false>(p, s);
+}
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int EPI = kStore>
+int launch_pp(const GemmArgs& p, hipStream_t s) {
+  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, kGemmWaves, 32, EPI, true>(p, s);
 }
 
 }  // namespace
 
 constexpr int kDmaBM = 256, kDmaBN = 256;
+
+// Fills in the dividers of the tile-id arithmetic; false when the ids would not fit 31 bits.
+// rows_of_tiles: upper bound of the number of tile rows (M-tiles, or groups x tiles_i for wgrad).
+static bool prepare_tile_ids(GemmArgs& p, int64_t rows_of_tiles) {
+  if (p.tiles_j <= 0 || rows_of_tiles * p.tiles_j >= (int64_t(1) << 31) - 8 * int64_t(p.tiles_j)) return false;
+  p.div_j = FastDivider(uint32_t(p.tiles_j));
+  p.div_i = FastDivider(uint32_t(p.tiles_i > 0 ? p.tiles_i : 1));
+  return true;
+}
 
 // rows form; returns STM_ERR_UNSUPPORTED when the shape does not fit these kernels.
 int launch_dma_rows(int dtype, const GemmArgs& base, const int32_t* offsets, int n_groups, int64_t m_cap, int b_is_nk,
@@ -961,6 +1125,14 @@ int launch_dma_rows(int dtype, const GemmArgs& base, const int32_t* offsets, int
   const int st = build_tile_table(offsets, n_groups, kDmaBM, m_cap, ws, s);
   if (st != STM_OK) return st;
   p.tiles_j = (p.n_j + kDmaBN - 1) / kDmaBN;
+  if (!prepare_tile_ids(p, max_m_tiles(m_cap, n_groups, kDmaBM))) return STM_ERR_UNSUPPORTED;
+  if (use_pingpong(b_is_nk ? kRowsFwd : kRowsDgrad)) {
+    if (dtype == STM_BF16)
+      return b_is_nk ? launch_pp<bf16_t, kDmaBM, kDmaBN, false, false, false>(p, s)
+                     : launch_pp<bf16_t, kDmaBM, kDmaBN, false, true, false>(p, s);
+    return b_is_nk ? launch_pp<f16_t, kDmaBM, kDmaBN, false, false, false>(p, s)
+                   : launch_pp<f16_t, kDmaBM, kDmaBN, false, true, false>(p, s);
+  }
   // Both operands K-contiguous (forward): stages of 64, so that every load moves full 128-byte
   // lines; a K-major operand in play (dgrad): four stages of 32 hide more latency.
   const bool deep = !b_is_nk || p.n_k % 64 != 0;
@@ -985,6 +1157,11 @@ int launch_dma_swiglu_fwd(int dtype, const GemmArgs& base, const int32_t* offset
   const int st = build_tile_table(offsets, n_groups, kDmaBM, m_cap, ws, s);
   if (st != STM_OK) return st;
   p.tiles_j = (p.ffn + kDmaBN / 2 - 1) / (kDmaBN / 2);
+  if (!prepare_tile_ids(p, max_m_tiles(m_cap, n_groups, kDmaBM))) return STM_ERR_UNSUPPORTED;
+  if (use_pingpong(kFusedFwd)) {
+    if (dtype == STM_BF16) return launch_pp<bf16_t, kDmaBM, kDmaBN, false, false, false, kSwigluFwd>(p, s);
+    return launch_pp<f16_t, kDmaBM, kDmaBN, false, false, false, kSwigluFwd>(p, s);
+  }
   const bool deep = p.n_k % 64 != 0;
   if (dtype == STM_BF16)
     return deep ? launch<bf16_t, kDmaBM, kDmaBN, false, false, false, 32, kSwigluFwd>(p, s)
@@ -1005,6 +1182,11 @@ int launch_dma_swiglu_bwd(int dtype, const GemmArgs& base, const int32_t* offset
   if (st != STM_OK) return st;
   p.n_j = p.ffn;
   p.tiles_j = (p.ffn + kDmaBN - 1) / kDmaBN;
+  if (!prepare_tile_ids(p, max_m_tiles(m_cap, n_groups, kDmaBM))) return STM_ERR_UNSUPPORTED;
+  if (use_pingpong(kFusedBwd)) {
+    if (dtype == STM_BF16) return launch_pp<bf16_t, kDmaBM, kDmaBN, false, true, false, kSwigluBwd>(p, s);
+    return launch_pp<f16_t, kDmaBM, kDmaBN, false, true, false, kSwigluBwd>(p, s);
+  }
   if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, false, true, false, 32, kSwigluBwd>(p, s);
   return launch<f16_t, kDmaBM, kDmaBN, false, true, false, 32, kSwigluBwd>(p, s);
 }
@@ -1024,6 +1206,7 @@ int launch_dma_fp8(int out_dtype, const GemmArgs& base, const int32_t* offsets, 
   const int st = build_tile_table(offsets, n_groups, kDmaBM, m_cap, ws, s);
   if (st != STM_OK) return st;
   p.tiles_j = (p.n_j + kDmaBN - 1) / kDmaBN;
+  if (!prepare_tile_ids(p, max_m_tiles(m_cap, n_groups, kDmaBM))) return STM_ERR_UNSUPPORTED;
   if (out_dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, false, false, false, 64, kStoreFp8>(p, s);
   return launch<f16_t, kDmaBM, kDmaBN, false, false, false, 64, kStoreFp8>(p, s);
 }
@@ -1037,6 +1220,15 @@ int launch_dma_wgrad(int dtype, const GemmArgs& base, int n_groups, int64_t m_ca
   p.tiles_i = (p.n_i + kDmaBM - 1) / kDmaBM;
   p.tiles_j = (p.n_j + kDmaBN - 1) / kDmaBN;
   p.n_groups = n_groups;
+  if (!prepare_tile_ids(p, int64_t(n_groups) * p.tiles_i)) return STM_ERR_UNSUPPORTED;
+  if (use_pingpong(kWgrad)) {
+    if (accumulate) {
+      if (dtype == STM_BF16) return launch_pp<bf16_t, kDmaBM, kDmaBN, true, true, true, kAccumF32>(p, s);
+      return launch_pp<f16_t, kDmaBM, kDmaBN, true, true, true, kAccumF32>(p, s);
+    }
+    if (dtype == STM_BF16) return launch_pp<bf16_t, kDmaBM, kDmaBN, true, true, true>(p, s);
+    return launch_pp<f16_t, kDmaBM, kDmaBN, true, true, true>(p, s);
+  }
   if (accumulate) {
     if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, true, true, true, 32, kAccumF32>(p, s);
     return launch<f16_t, kDmaBM, kDmaBN, true, true, true, 32, kAccumF32>(p, s);

@@ -475,7 +475,8 @@ def test_nothing_routed_early_out_keeps_the_tail_and_leaves_routed_batches_alone
     shared = torch.randn(T, H, generator=gen).bfloat16().to(DEV)
     none = torch.full((T, K), -1, dtype=torch.int64, device=DEV)
     out = M.hip_routed_grouped_ffn(w1, w2, swiglu, x, none, tw, out_scale=2.5, out_addend=shared)
-    assert torch.equal(out, (x * tw.sum()) * 2.5 + shared)
+    # (the kernel's sum of the weights and torch's differ in the order of their fp32 additions)
+    assert rel_l2(out, (x * tw.sum()) * 2.5 + shared) <= 4e-3
     one = none.clone()
     one[5, 1] = 2  # a single routed slot: the early-out must not fire
     out = M.hip_routed_grouped_ffn(w1, w2, swiglu, x, one, tw)
