@@ -39,7 +39,8 @@ enum {
   STM_ERR_ARG = -1,         /* null pointer, negative size, inconsistent shapes   */
   STM_ERR_UNSUPPORTED = -2, /* dtype / size outside what the kernels implement    */
   STM_ERR_WORKSPACE = -3,   /* workspace smaller than *_workspace_bytes() said    */
-  STM_ERR_LAUNCH = -4       /* the HIP runtime refused the launch                 */
+  STM_ERR_LAUNCH = -4,      /* the HIP runtime refused the launch                 */
+  STM_ERR_CAPACITY = -5     /* problem larger than the library's static scratch   */
 };
 
 /* Device-side status words, int32[STM_STATUS_WORDS], written by the routing and
@@ -88,6 +89,22 @@ int stm_index_compute(const void* ids, int ids_are_i64, int64_t n_slots, int n_e
 int stm_route_plan(const void* ids, int ids_are_i64, int64_t n_slots, int n_experts, int32_t* hist_out,
                    int32_t* offsets_out, int32_t* pos_out, int32_t* status, void* workspace, size_t workspace_bytes,
                    stm_stream_t stream);
+
+/* stm_route_plan for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same outputs as stm_route_plan, bit for bit; the counter rows live in a
+ * device array owned by the library (one copy per GPU, stm_route_plan_static_capacity_bytes()
+ * = 2 MiB, held until the process ends) instead of a caller workspace, and the call
+ * itself allocates and frees nothing.  A problem with
+ * stm_route_workspace_bytes(n_slots, n_experts) above the capacity (more than about
+ * 2^19 counter cells = ceil(n_slots / 256) * n_experts) returns STM_ERR_CAPACITY and
+ * launches nothing.  All calls on one GPU share that GPU's array: calls that overlap
+ * in time on one GPU (different streams, different threads) race; order them.  The first
+ * call on a device looks the array's address up (no allocation, but make that call outside
+ * a graph capture). */
+size_t stm_route_plan_static_capacity_bytes(void);
+int stm_route_plan_static(const void* ids, int ids_are_i64, int64_t n_slots, int n_experts, int32_t* hist_out,
+                          int32_t* offsets_out, int32_t* pos_out, int32_t* status, stm_stream_t stream);
 
 /* int64/int32 group sizes -> int32 offsets [G+1] (grouped_gemm's batch_sizes,
  * moe_utils.py:443-453). */

@@ -40,6 +40,8 @@ SIGNATURES = {
     "stm_histogram": (I, [P, I, L, I, P, P, P, Z, P]),
     "stm_index_compute": (I, [P, I, L, I, P, I, P, P, P, Z, P]),
     "stm_route_plan": (I, [P, I, L, I, P, P, P, P, P, Z, P]),
+    "stm_route_plan_static_capacity_bytes": (Z, []),
+    "stm_route_plan_static": (I, [P, I, L, I, P, P, P, P, P]),
     "stm_group_offsets": (I, [P, I, I, P, P]),
     "stm_permute_fwd": (I, [P, P, I, P, L, I, L, L, P, P]),
     "stm_zero_unwritten_rows": (I, [P, P, L, L, P]),

@@ -12,6 +12,7 @@ const char* stm_status_string(int status) {
     case STM_ERR_UNSUPPORTED: return "unsupported dtype or size";
     case STM_ERR_WORKSPACE: return "workspace too small";
     case STM_ERR_LAUNCH: return "HIP launch failed";
+    case STM_ERR_CAPACITY: return "problem exceeds the capacity of the library's static scratch array";
     default: return "unknown status";
   }
 }

@@ -13,6 +13,8 @@
 //   index kernel : replays the ranking, starting every counter from the scanned table
 //
 // Everything is integer arithmetic, so results are bit-reproducible.
+#include <atomic>
+
 #include "common.hpp"
 
 namespace stm {
@@ -367,6 +369,36 @@ int sort_slots_by_row(const void* pos, int pos_is_i64, int64_t n_slots, int64_t 
 
 }  // namespace stm
 
+namespace stm {
+namespace {
+
+// Counter rows of stm_route_plan_static: device memory owned by the library, one copy per GPU,
+// held until the process ends.  Host code never uses the array's name as an address: the
+// device address is looked up once per device and kept.
+constexpr size_t kStaticScratchBytes = size_t(2) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> scratch_address[kMaxDevices];
+
+// Device address of `scratch` on the current device (nullptr on failure).
+void* static_scratch() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void* p = scratch_address[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  void* looked_up = nullptr;
+  if (hipGetSymbolAddress(&looked_up, HIP_SYMBOL(scratch)) != hipSuccess || !looked_up) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  scratch_address[dev].store(looked_up, std::memory_order_release);
+  return looked_up;
+}
+
+}  // namespace
+}  // namespace stm
+
 extern "C" {
 
 size_t stm_route_workspace_bytes(int64_t n_slots, int n_experts) {
@@ -398,6 +430,22 @@ int stm_route_plan(const void* ids, int ids_are_i64, int64_t n_slots, int n_expe
   if (!offsets_out || (n_slots > 0 && !pos_out)) return STM_ERR_ARG;
   return stm::run_sort(ids, ids_are_i64, n_slots, n_experts, nullptr, 0, hist_out, offsets_out, pos_out, status,
                        workspace, workspace_bytes, stm::as_stream(stream));
+}
+
+size_t stm_route_plan_static_capacity_bytes(void) { return stm::kStaticScratchBytes; }
+
+int stm_route_plan_static(const void* ids, int ids_are_i64, int64_t n_slots, int n_experts, int32_t* hist_out,
+                          int32_t* offsets_out, int32_t* pos_out, int32_t* status, stm_stream_t stream) {
+  if (!offsets_out || (n_slots > 0 && !pos_out)) return STM_ERR_ARG;
+  if (n_slots < 0 || n_experts < 0) return STM_ERR_ARG;
+  const size_t need = stm_route_workspace_bytes(n_slots, n_experts);
+  if (need > stm::kStaticScratchBytes) return STM_ERR_CAPACITY;
+  void* ws = stm::static_scratch();
+  if (!ws) return STM_ERR_LAUNCH;
+  // every counter cell the scan reads is first written by the count kernel of the same call, so
+  // what an earlier (larger) call left in the array is never seen
+  return stm::run_sort(ids, ids_are_i64, n_slots, n_experts, nullptr, 0, hist_out, offsets_out, pos_out, status, ws,
+                       stm::kStaticScratchBytes, stm::as_stream(stream));
 }
 
 int stm_group_offsets(const void* sizes, int sizes_are_i64, int n_groups, int32_t* offsets_out, stm_stream_t stream) {
