@@ -38,8 +38,13 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 # HBM bytes per grouped-GEMM launch (fetched + written, mean over the six launches of a step),
 # from hardware counters collected in separate profiler runs of this script (FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB copies of
-# --traffic-probe); the summaries of those runs are kept under profiles/.  None = not measured.
-MEASURED_GEMM_TRAFFIC_BYTES = {"c2": 2.48e9, "c3": None, "c4": None}
+# --traffic-probe).  Each figure names the summary under profiles/ it was taken from and holds
+# for the kernels of that summary only: None = not measured for the kernels as they are now.
+MEASURED_GEMM_TRAFFIC = {
+    "c2": {"bytes": None, "source": "profiles/persistent_gemm_c2_hbm_traffic.txt"},
+    "c3": {"bytes": None, "source": None},
+    "c4": {"bytes": None, "source": None},
+}
 
 WORKLOADS = {
     "c1": dict(T=4096, H=1024, E=8, K=2, F=2048, sigmoid=False, norm=False, n_group=1, topk_group=1, std=0.02, dtype="fp32"),
@@ -87,13 +92,13 @@ def make_inputs(cfg, seed, device):
 
 
 def cpu_baseline(cfg, seed, threads):
-    """Oracle on CPU tensors, fp32, on a bounded sample of the same workload: an eighth of
-    the tokens over all experts (the per-expert matmul loop at 1/8 of the rows per expert),
-    passes repeated until about 12 s have gone by (two or three passes)."""
+    """Oracle on CPU tensors, fp32, on a bounded sample of the same workload: a sixteenth of
+    the tokens over all experts (the per-expert matmul loop at 1/16 of the rows per expert), one
+    warm-up pass and two timed ones."""
     from oracle import moe_oracle as O
 
     torch.set_num_threads(threads)
-    T = cfg["T"] // 8
+    T = cfg["T"] // 16
     H, E, F, K = cfg["H"], cfg["E"], cfg["F"], cfg["K"]
     gen = torch.Generator().manual_seed(seed)
     x = (torch.randn(T, H, generator=gen) * cfg["std"]).bfloat16().float().requires_grad_(True)
@@ -103,7 +108,7 @@ def cpu_baseline(cfg, seed, threads):
     go = torch.randn(T, H, generator=gen)
     flops = 6.0 * T * K * H * 3 * F
     times = []
-    for it in range(3):  # first pass doubles as the warm-up when time is short
+    for it in range(3):  # pass 0 is the warm-up
         for t in (x, w1, w2, logits):
             t.grad = None
         t0 = time.perf_counter()
@@ -113,16 +118,16 @@ def cpu_baseline(cfg, seed, threads):
         )  # fmt: skip
         out.backward(go)
         times.append(time.perf_counter() - t0)
-        if sum(times) > 12.0:
-            break
-    best = min(times)
+    timed = times[1:]
+    mean = sum(timed) / len(timed)
     return {
-        "value": flops / best / 1e12,
+        "value": flops / mean / 1e12,
         "unit": "TFLOP/s",
         "cores": threads,
+        "host_cores": os.cpu_count(),
         "kind": "port",
-        "sample": f"{T} of {cfg['T']} tokens over all {E} experts, fp32, fwd+bwd, best of {len(times)} passes, "
-        f"{best * 1e3:.0f} ms per pass",
+        "sample": f"{T} of {cfg['T']} tokens over all {E} experts, fp32, fwd+bwd, 1 warm-up + {len(timed)} timed passes "
+        f"(mean {mean * 1e3:.0f} ms, warm-up {times[0] * 1e3:.0f} ms) on {threads} threads of {os.cpu_count()} host cores",
     }
 
 
@@ -142,19 +147,18 @@ def cpu_baseline_fwd_dgrad(cfg, seed, threads):
     sizes = torch.full((E,), rows_per, dtype=torch.int64)
     flops = 4.0 * E * rows_per * H * 3 * F
     times = []
-    for _ in range(3):
+    for _ in range(3):  # pass 0 is the warm-up
         x.grad = None
         t0 = time.perf_counter()
         y = O.grouped_gemm(O.swiglu(O.grouped_gemm(x, w1, sizes, trans_b=True)), w2, sizes, trans_b=True)
         y.backward(go)
         times.append(time.perf_counter() - t0)
-        if sum(times) > 12.0:
-            break
-    best = min(times)
+    timed = times[1:]
+    mean = sum(timed) / len(timed)
     return {
-        "value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-        "sample": f"{E} of {cfg['E']} experts at {rows_per} rows each, fp32, forward + input gradient, best of "
-        f"{len(times)} passes, {best * 1e3:.0f} ms per pass",
+        "value": flops / mean / 1e12, "unit": "TFLOP/s", "cores": threads, "host_cores": os.cpu_count(), "kind": "port",
+        "sample": f"{E} of {cfg['E']} experts at {rows_per} rows each, fp32, forward + input gradient, 1 warm-up + "
+        f"{len(timed)} timed passes (mean {mean * 1e3:.0f} ms) on {threads} threads of {os.cpu_count()} host cores",
     }  # fmt: skip
 
 
@@ -315,19 +319,45 @@ def main():
     flops_per_launch = flops / 6.0
     avg_launch_ms = gemm_ms / max(gemm_calls, 1)
     achieved = flops_per_launch / (avg_launch_ms * 1e-3) / 1e12 if gemm_calls else 0.0
-    roofline = {
-        "bound": "mfma",
-        "kernel": "generic_gemm_kernel (fp32 FMA tiles; priced against the fp32 MFMA peak)" if fp32
-        else "persistent_gemm_kernel (grouped GEMM fwd / dgrad / wgrad, 256x256 tiles, SwiGLU in two epilogues)",
-        "achieved": achieved,
-        "peak": peak,
-        "unit": "TFLOP/s",
-        "frac": achieved / peak,
-        "traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(args.workload),
-        "flops_per_launch": flops_per_launch,
-        "avg_launch_us": avg_launch_ms * 1e3,
+    # Compulsory HBM bytes of the six launches (every operand read once, every output written
+    # once; gate_up, h and d gate_up as the fused kernels move them), mean per launch.  A launch is
+    # priced against whichever roof binds: the matrix peak, or HBM when streaming the operands
+    # takes longer than the arithmetic (few rows per expert: the large-expert workload).
+    w_elems, act = 3.0 * E * F * H, float(N)
+    step_bytes = e * (
+        (act * H + w_elems * 2 / 3 + act * 3 * F)  # forward 1 + SwiGLU: x rows, w1 -> gate_up, h
+        + (act * F + w_elems / 3 + act * H)  # forward 2: h, w2 -> y
+        + (act * H + w_elems / 3 + act * 2 * F + act * 2 * F)  # dgrad 2 + SwiGLU backward: d y, w2, gate_up -> d gate_up
+        + (act * 2 * F + w_elems * 2 / 3 + act * H)  # dgrad 1: d gate_up, w1 -> d x rows
+        + (act * H + act * F + w_elems / 3)  # wgrad 2
+        + (act * 2 * F + act * H + w_elems * 2 / 3)  # wgrad 1
+    )
+    bytes_per_launch = step_bytes / 6.0
+    t_flop_ms = flops_per_launch / (peak * 1e12) * 1e3
+    t_bytes_ms = bytes_per_launch / (PEAK_HBM_GBPS * 1e9) * 1e3
+    hbm_bound = t_bytes_ms > t_flop_ms
+    measured = MEASURED_GEMM_TRAFFIC.get(args.workload, {"bytes": None, "source": None})
+    kernel_name = (
+        "generic_gemm_kernel (fp32 FMA tiles; priced against the fp32 MFMA peak)" if fp32
+        else "persistent_gemm_kernel (grouped GEMM fwd / dgrad / wgrad, 256x256 tiles, SwiGLU in two epilogues)"
+    )
+    if hbm_bound and gemm_calls:
+        gbps = bytes_per_launch / (avg_launch_ms * 1e-3) / 1e9
+        roofline = {
+            "bound": "hbm", "kernel": kernel_name, "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+            "frac": gbps / PEAK_HBM_GBPS, "matrix_TFLOP/s": achieved, "frac_of_mfma_peak": achieved / peak,
+        }  # fmt: skip
+    else:
+        roofline = {
+            "bound": "mfma", "kernel": kernel_name, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+            "frac": achieved / peak,
+        }  # fmt: skip
+    roofline.update({
+        "traffic": measured["bytes"], "traffic_source": measured["source"] if measured["bytes"] else None,
+        "flops_per_launch": flops_per_launch, "algorithmic_bytes_per_launch": bytes_per_launch,
+        "roof_ms_per_launch": {"mfma": t_flop_ms, "hbm": t_bytes_ms}, "avg_launch_us": avg_launch_ms * 1e3,
         "launches_per_step": gemm_calls / args.steps,
-    }
+    })  # fmt: skip
 
     # The stand-alone combine op (moe_weighted_gather, weights applied in the combine), outside
     # the timed steps: the fused FFN's backward replaces its backward kernel by a row copy.
@@ -399,7 +429,7 @@ def main():
         "entry_avg_us": entry_us,
     }
     if not args.no_cpu_baseline:
-        threads = min(os.cpu_count() or 1, 16)
+        threads = min(os.cpu_count() or 1, 16)  # the box's CPU share is 16 cores whatever the host shows
         result["cpu_baseline"] = cpu_baseline(cfg, args.seed, threads)
     print(json.dumps(result))
 
