@@ -163,35 +163,32 @@ def cpu_baseline_fwd_dgrad(cfg, seed, threads):
 
 
 def run_fp8(args, cfg):
-    """Workload c5: the expert FFN of c4 on e4m3 operands (weights quantised once, activations on the
-    way into each GEMM), forward + dgrad over the rows the seeded router sends to each expert."""
+    """Workload c5: the c4 layer with the expert GEMMs on e4m3 operands (``settings.fp8_experts``):
+    router, then ``routed_grouped_ffn`` forward and its input gradients (weights quantised once,
+    activations on the way into each GEMM; no weight gradients, as the workload is defined)."""
+    from steptronoss_amd.model.common.feed_forward import swiglu
     from steptronoss_amd.model.common.moe_block import forward_router
-    from steptronoss_amd.model.utils.fp8 import Fp8ExpertFFN
-    from steptronoss_amd.model.utils.moe_utils import histogram, index_compute, moe_scatter
+    from steptronoss_amd.model.utils import moe_utils as M
     from steptronoss_amd.profiling import KernelTimer
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    bf16_cfg = dict(cfg, dtype="bf16")
-    x, w1, w2, logits, go = make_inputs(bf16_cfg, args.seed, dev)
+    x, w1, w2, logits, go = make_inputs(dict(cfg, dtype="bf16"), args.seed, dev)
     T, H, E, K, F = cfg["T"], cfg["H"], cfg["E"], cfg["K"], cfg["F"]
     N = T * K
-    ids, _w, _aux, _h = forward_router(
-        logits, K, use_sigmoid=cfg["sigmoid"], norm_expert_weight=cfg["norm"], n_group=cfg["n_group"],
-        topk_group=cfg["topk_group"],
-    )  # fmt: skip
-    sizes = histogram(ids, E)
-    pos = index_compute(ids, sizes)
-    rows = moe_scatter(x, pos).contiguous()
-    grad_rows = moe_scatter(go, pos).contiguous()
-    sizes = sizes.to(torch.int64)
-    ffn = Fp8ExpertFFN(w1, w2)
-    del w1, w2, x, go, logits
-    torch.cuda.empty_cache()
+    x.requires_grad_(True)
+    logits.requires_grad_(True)
+    one = torch.ones((), device=dev)
+    M.settings.fp8_experts = True
 
     def step():
-        y, gate_up = ffn.forward_rows(rows, sizes)
-        return ffn.dgrad_rows(grad_rows, gate_up, sizes), y
+        x.grad = logits.grad = None
+        ids, weights, aux, _hist = forward_router(
+            logits, K, use_sigmoid=cfg["sigmoid"], norm_expert_weight=cfg["norm"], n_group=cfg["n_group"],
+            topk_group=cfg["topk_group"],
+        )  # fmt: skip
+        out = M.hip_routed_grouped_ffn(w1, w2, swiglu, x, ids, weights)
+        torch.autograd.backward([out, aux], [go, one * 0.01])
 
     for _ in range(args.warmup):
         step()
@@ -207,6 +204,10 @@ def run_fp8(args, cfg):
     timing = kt.summary()
     gemm = timing["stm_grouped_gemm_fp8_pow2"]
     achieved = (flops / 4.0) / (gemm["avg_us"] * 1e-6) / 1e12
+    # per launch (mean of the four): codes of the rows and of one weight orientation in, bf16 rows out
+    bytes_per_launch = (N * (H + 2 * F + F + H) + 2.0 * 3 * E * F * H + 2.0 * N * (2 * F + H + F + H)) / 4.0
+    t_flop_ms = flops / 4.0 / (PEAK_FP8_TFLOPS * 1e12) * 1e3
+    t_bytes_ms = bytes_per_launch / (PEAK_HBM_GBPS * 1e9) * 1e3
     quant = timing["stm_quantize_e4m3_1x128_pow2"]
     quant_bytes = (N * H * 3 + N * 2 * F * 3 + N * F * 3 + N * H * 3) / 4.0  # bf16 in, codes out, mean of the four
     result = {
@@ -214,16 +215,18 @@ def run_fp8(args, cfg):
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3", "data": "synthetic",
         "config": {
-            "workload": f"c5: expert FFN of the c4 layer (T={T} H={H} E={E} top-{K} F={F}) on e4m3 operands with one "
-            "power-of-two scale per row and 128 elements, bf16 outputs; forward + dgrad over the routed rows "
-            "(weights quantised once, activations on the way into each GEMM)",
+            "workload": f"c5: MoE layer T={T} H={H} E={E} top-{K} F={F}, sigmoid group-limited routing, expert GEMMs on "
+            "e4m3 operands with one power-of-two scale per row and 128 elements (bf16 outputs) through routed_grouped_ffn; "
+            "router + forward + input gradients",
             "tokens": T, "hidden": H, "experts": E, "top_k": K, "expert_ffn": F, "seed": args.seed,
         },
         "frac_of_mfma_peak": flops / (ms_per_step * 1e-3) / 1e12 / PEAK_FP8_TFLOPS,
         "roofline": {
-            "bound": "mfma", "kernel": "persistent_gemm_kernel, e4m3 operands on v_mfma_scale_f32_32x32x64_f8f6f4",
+            "bound": "hbm" if t_bytes_ms > t_flop_ms else "mfma",
+            "kernel": "persistent_gemm_kernel, e4m3 operands on v_mfma_scale_f32_32x32x64_f8f6f4",
             "achieved": achieved, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_FP8_TFLOPS,
-            "traffic": None, "flops_per_launch": flops / 4.0, "avg_launch_us": gemm["avg_us"],
+            "traffic": None, "flops_per_launch": flops / 4.0, "algorithmic_bytes_per_launch": bytes_per_launch,
+            "roof_ms_per_launch": {"mfma": t_flop_ms, "hbm": t_bytes_ms}, "avg_launch_us": gemm["avg_us"],
             "launches_per_step": gemm["calls"] / args.steps,
         },
         "bandwidth": {

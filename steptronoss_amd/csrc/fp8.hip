@@ -70,18 +70,35 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(const T* __restrict__
   float amax = 0.f;
 #pragma unroll
   for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[e]));
-#pragma unroll
-  for (int off = 8; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, kWave));
+  // the largest magnitude of the 16 lanes of this block: four rotations inside the 16-lane row
+  // (row_ror 8, 4, 2, 1 on the data-parallel path; every lane ends up with the maximum)
+#define STM_ROW_ROR_MAX(CTRL) \
+  amax = fmaxf(amax, __builtin_bit_cast(float, dpp_move<CTRL, 0xf>(0, __builtin_bit_cast(int, amax))))
+  STM_ROW_ROR_MAX(0x128);
+  STM_ROW_ROR_MAX(0x124);
+  STM_ROW_ROR_MAX(0x122);
+  STM_ROW_ROR_MAX(0x121);
+#undef STM_ROW_ROR_MAX
   const float scale = block_scale<POW2>(amax);
   if (live && sub == 0) scales[POW2 ? b * rows + r : r * n_blocks + b] = scale;
   if (in) {
-    uint32_t lo = 0, hi = 0;
+    float q[8];
+    if constexpr (POW2) {
+      // 1 / 2^e as a bit pattern: the product is the exact quotient
+      const float inv = __uint_as_float(0x7f000000u - __float_as_uint(scale));
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      lo |= e4m3_code(v[e] / scale) << (8 * e);
-      hi |= e4m3_code(v[4 + e] / scale) << (8 * e);
+      for (int e = 0; e < 8; ++e) q[e] = v[e] * inv;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) q[e] = v[e] / scale;
     }
-    *reinterpret_cast<uint2*>(codes + r * cols + c0) = make_uint2(lo, hi);
+    // the hardware conversion (OCP e4m3 on gfx950: nearest even, subnormals kept); |q| <= 448
+    int lo = 0, hi = 0;
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], lo, false);
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], lo, true);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], hi, false);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], hi, true);
+    *reinterpret_cast<uint2*>(codes + r * cols + c0) = make_uint2(uint32_t(lo), uint32_t(hi));
   }
 }
 

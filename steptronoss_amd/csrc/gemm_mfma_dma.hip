@@ -1080,9 +1080,9 @@ constexpr int kGemmWaves = 8;
 
 // Two schedules of the main loop exist: "interleaved" (every wave mixes its LDS reads and loads
 // into its own MFMAs; stages of 64 when both operands are K-contiguous) and "ping-pong".  Each
-// product runs the one measured faster for it on the expert-FFN shapes: ping-pong for the weight
-// gradients and the fused SwiGLU forward (its epilogue runs under the partner wave's MFMAs),
-// interleaved for the rest.  STM_GEMM_SCHEDULE=interleaved / pingpong forces one for all.
+// product runs the one measured faster for it on the expert-FFN shapes (they are within a few per
+// cent of each other everywhere): ping-pong for the weight gradients, interleaved for the rest.
+// STM_GEMM_SCHEDULE=interleaved / pingpong forces one for all.
 enum Product { kRowsFwd, kRowsDgrad, kFusedFwd, kFusedBwd, kWgrad };
 bool use_pingpong(Product which) {
   static const int forced = [] {
@@ -1090,7 +1090,7 @@ bool use_pingpong(Product which) {
     return !v ? 0 : v[0] == 'i' ? 1 : v[0] == 'p' ? 2 : 0;
   }();
   if (forced) return forced == 2;
-  return which == kWgrad || which == kFusedFwd;
+  return which == kWgrad;
 }
 
 template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int BK, int EPI = kStore>

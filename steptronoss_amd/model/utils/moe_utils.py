@@ -59,6 +59,12 @@ class Settings:
     probe_activation: ``routed_grouped_ffn`` fuses the SwiGLU into the GEMMs only for an
         activation it knows by identity; with this switch a callable that merely behaves like the
         SwiGLU on a probe tensor is replaced as well (and a warning is logged).
+    fp8_experts: ``routed_grouped_ffn`` (bf16 / fp16 tensors, SwiGLU known by identity, hidden and
+        ffn sizes multiples of 128, at least 4096 slots) runs the two expert GEMMs and their input
+        gradients on e4m3 operands with one power-of-two scale per row and 128 contraction elements
+        (the fp8 benchmark configuration; no counterpart in the reference): activations are quantised
+        on the way into each GEMM, the weights once per weight version, in both orientations.
+        Weight gradients stay in the tensors' own dtype.
     deferred_id_check: ``routed_grouped_ffn`` copies the routing status words to pinned host
         memory without waiting; a later call (or ``check_deferred_status()``) that finds such a
         copy complete raises the reference's "out-of-range" ``ValueError`` for an expert id
@@ -71,6 +77,7 @@ class Settings:
     fuse_main_grad: bool = False
     probe_activation: bool = False
     deferred_id_check: bool = True
+    fp8_experts: bool = False
 
 
 settings = Settings()
@@ -778,6 +785,105 @@ class _FusedRoutedFFN(torch.autograd.Function):
         return gw1, gw2, gx, None, (gtw if need_tw else None), None, None, (grad_out if need_addend else None)
 
 
+_FP8_WEIGHTS: dict = {}
+
+
+def _fp8_weights(w1: torch.Tensor, w2: torch.Tensor, swiglu_limit):
+    """The quantised copies of the expert weights, re-made when a weight was written to (its
+    version counter moved) or replaced."""
+    from steptronoss_amd.model.utils.fp8 import Fp8ExpertFFN
+
+    key = (w1.data_ptr(), w2.data_ptr(), tuple(w1.shape), tuple(w2.shape), w1.dtype)
+    stamp = (w1._version, w2._version, swiglu_limit)
+    hit = _FP8_WEIGHTS.get(key)
+    if hit is None or hit[0] != stamp:
+        _FP8_WEIGHTS.clear()  # one layer's copies at a time: they are as large as the weights
+        hit = _FP8_WEIGHTS[key] = (stamp, Fp8ExpertFFN(w1.detach(), w2.detach(), swiglu_limit))
+    return hit[1]
+
+
+class _Fp8RoutedFFN(torch.autograd.Function):
+    """``routed_grouped_ffn`` with the expert GEMMs (forward and input gradients) on e4m3 operands.
+    Same data flow as the unfused bf16 path: permute, GEMM, SwiGLU, GEMM, weighted combine; every
+    GEMM input is quantised by ``stm_quantize_e4m3_1x128_pow2`` right before it is used."""
+
+    @staticmethod
+    def forward(ctx, w1, w2, x, token_expert_ids, token_weights, swiglu_limit, out_scale=None, out_addend=None):
+        from steptronoss_amd.model.common.feed_forward import swiglu_fwd_rows
+        from steptronoss_amd.model.utils.fp8 import grouped_gemm_fp8_pow2_rows, quantize_e4m3_1x128_pow2
+
+        dev = x.device
+        T, H = x.shape
+        K = token_expert_ids.shape[1]
+        E = w1.shape[0]
+        n_rows = T * K
+        with torch.cuda.device(dev):
+            ffn = _fp8_weights(w1, w2, swiglu_limit)
+            _hist, offsets, pos, status = route_plan(token_expert_ids, E)
+            if settings.validate_fused:
+                if int(status[_lib.ST_ID_OUT_OF_RANGE]):
+                    raise ValueError("top_k_rank contains out-of-range expert index")
+            elif settings.deferred_id_check:
+                _defer_status_check(status)
+            live = offsets[E:]
+            xp = torch.zeros((n_rows, H), device=dev, dtype=x.dtype)  # (unused rows are quantised too: keep them finite)
+            call("stm_permute_fwd", ptr(x), ptr(pos), 0, ptr(xp), T, K, H * x.element_size(), n_rows, None, stream())
+            q, sc = quantize_e4m3_1x128_pow2(xp)
+            gu = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w1_q, ffn.w1_s, offsets, x.dtype)
+            h = swiglu_fwd_rows(gu, swiglu_limit, live)
+            q, sc = quantize_e4m3_1x128_pow2(h)
+            y = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w2_q, ffn.w2_s, offsets, x.dtype)
+            addend = None if out_addend is None else out_addend.contiguous()
+            out = _combine_rows(y, pos, token_weights, out_scale, addend)
+            _nothing_routed_fwd(live, x, token_weights, out, out_scale, addend)
+        ctx.save_for_backward(w1, w2, x, xp, gu, h, y, pos, offsets, token_weights)
+        ctx.ffn = ffn
+        ctx.limit = swiglu_limit
+        ctx.out_scale = out_scale
+        ctx.shape = (T, H, K, E)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from steptronoss_amd.model.common.feed_forward import swiglu_bwd_rows
+        from steptronoss_amd.model.utils.fp8 import grouped_gemm_fp8_pow2_rows, quantize_e4m3_1x128_pow2
+
+        w1, w2, x, xp, gu, h, y, pos, offsets, token_weights = ctx.saved_tensors
+        T, H, K, E = ctx.shape
+        ffn = ctx.ffn
+        dev = grad_out.device
+        need_w1, need_w2, need_x, _, need_tw, _, _, need_addend = ctx.needs_input_grad
+        gw1 = gw2 = gx = None
+        with torch.cuda.device(dev):
+            live = offsets[E:]
+            go = grad_out.contiguous()
+            gy = torch.zeros_like(y)
+            gtw = _combine_rows_bwd(go, y, pos, token_weights, gy, None, ctx.out_scale)
+            if need_w2:
+                gw2 = _gemm_wgrad(gy, h, offsets, E)
+            if need_w1 or need_x:
+                q, sc = quantize_e4m3_1x128_pow2(gy)
+                dh = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w2t_q, ffn.w2t_s, offsets, gy.dtype)
+                dgu = swiglu_bwd_rows(gu, dh, ctx.limit, live)
+                if need_w1:
+                    gw1 = _gemm_wgrad(dgu, xp, offsets, E)
+                if need_x:
+                    q, sc = quantize_e4m3_1x128_pow2(dgu)
+                    dxp = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w1t_q, ffn.w1t_s, offsets, gy.dtype)
+                    gx = _permute_rows_bwd(dxp, pos, H)
+            if need_x or need_tw:
+                _nothing_routed_bwd(live, go, x, token_weights, gx, gtw if need_tw else None, ctx.out_scale)
+        return gw1, gw2, gx, None, (gtw if need_tw else None), None, None, (grad_out if need_addend else None)
+
+
+def _fp8_takes(w1, w2, x, n_slots: int) -> bool:
+    H, F2 = x.shape[1], w1.shape[1]
+    return (
+        x.dtype in (torch.bfloat16, torch.float16) and H % 128 == 0 and F2 % 256 == 0 and n_slots >= 4096
+        and w1.shape[2] == H and w2.shape[1] == H and w2.shape[2] * 2 == F2
+    )  # fmt: skip
+
+
 _ACT_CACHE: dict = {}
 _REFERENCE_SWIGLU = ("steptronoss.model.common.feed_forward", "FeedForwardConfig.activation")
 
@@ -883,6 +989,8 @@ def hip_routed_grouped_ffn(w1, w2, act, x, token_expert_ids, token_weights, *, o
         if settings.deferred_id_check:
             check_deferred_status()
         fused, limit = _swiglu_limit_of(act, w1.shape[1], x.dtype, dev)
+        if fused and settings.fp8_experts and _fp8_takes(w1c, w2c, xc, T * K):
+            return _Fp8RoutedFFN.apply(w1c, w2c, xc, ids, tw, limit, out_scale, out_addend)
         if fused:
             return _FusedRoutedFFN.apply(w1c, w2c, xc, ids, tw, limit, out_scale, out_addend)
         _hist, offsets, pos, status = route_plan(ids, E)

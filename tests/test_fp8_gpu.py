@@ -185,3 +185,48 @@ def test_fp8_expert_ffn_forward_and_dgrad_against_the_fp32_layer():
     assert rel_l2(y, ref) <= 7.5e-2
     assert rel_l2(gx, xr.grad) <= 7.5e-2
     assert rel_l2(y, ref) >= 1e-3  # it is an fp8 result, not the bf16 path by another name
+
+
+def test_fp8_routed_ffn_through_the_operator_api():
+    """``settings.fp8_experts`` puts the expert GEMMs (forward and input gradients) of
+    ``routed_grouped_ffn`` on e4m3 operands; weight gradients stay bf16.  Against the fp32 oracle the
+    two chained fp8 GEMMs leave about sqrt(2) x 3.6 % (see the top of this file)."""
+    from steptronoss_amd.model.common.feed_forward import swiglu
+    from steptronoss_amd.model.utils import moe_utils as M
+    from steptronoss_amd.profiling import KernelTimer
+    from tests.helpers import make_topk_ids
+
+    gen = torch.Generator().manual_seed(41)
+    T, H, K, E, Fh = 1024, 256, 8, 16, 128
+    x = (torch.randn(T, H, generator=gen) * 0.5).bfloat16()
+    w1 = (torch.randn(E, 2 * Fh, H, generator=gen) * 0.1).bfloat16()
+    w2 = (torch.randn(E, H, Fh, generator=gen) * 0.1).bfloat16()
+    ids = make_topk_ids(T, K, E, gen=gen, invalid_frac=0.1)
+    tw = torch.rand(T, K, generator=gen)
+    go = torch.randn(T, H, generator=gen).bfloat16()
+    ref_in = [t.clone().float().requires_grad_(True) for t in (w1, w2, x, tw)]
+    O.routed_grouped_ffn(ref_in[0], ref_in[1], O.swiglu, ref_in[2], ids, ref_in[3]).backward(go.float())
+    ref_out = O.routed_grouped_ffn(ref_in[0], ref_in[1], O.swiglu, ref_in[2], ids, ref_in[3]).detach()
+    got_in = [t.to(DEV).requires_grad_(True) for t in (w1, w2, x, tw)]
+    old = M.settings.fp8_experts
+    try:
+        M.settings.fp8_experts = True
+        with KernelTimer() as kt:
+            out = M.routed_grouped_ffn(got_in[0], got_in[1], swiglu, got_in[2], ids.to(DEV), got_in[3])
+            out.backward(go.to(DEV))
+        assert kt.summary()["stm_grouped_gemm_fp8_pow2"]["calls"] == 4
+        # the weights are quantised once per version: a second call re-uses the codes, a write re-makes them
+        cached = M._fp8_weights(got_in[0], got_in[1], None)
+        M.routed_grouped_ffn(got_in[0], got_in[1], swiglu, got_in[2], ids.to(DEV), got_in[3])
+        assert M._fp8_weights(got_in[0], got_in[1], None) is cached
+        with torch.no_grad():
+            got_in[0].mul_(1.0)
+        assert M._fp8_weights(got_in[0], got_in[1], None) is not cached
+    finally:
+        M.settings.fp8_experts = old
+    errs = {"out": rel_l2(out, ref_out)}
+    for name, g, r in zip(("dw1", "dw2", "dx", "dtw"), got_in, ref_in):
+        errs[name] = rel_l2(g.grad, r.grad)
+    print("fp8 routed FFN against the fp32 oracle:", {k: f"{v:.3f}" for k, v in errs.items()})
+    assert max(errs.values()) <= 7.5e-2, errs
+    assert errs["out"] >= 1e-3  # it is an fp8 result, not the bf16 path by another name
