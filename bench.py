@@ -382,6 +382,28 @@ def main():
         timing.setdefault(name, t)
     del rows, slot_weights
 
+    # The gate GEMM folded into the router (outside the timed steps, which start from ready-made
+    # logits as the workload is defined): one kernel against library GEMM + router.
+    gate_us = {}
+    if not fp32:
+        from steptronoss_amd.model.common.moe_block import forward_gate_router
+
+        wg = (torch.randn(E, H, device=dev) * 0.02).to(x.dtype)
+        rk = dict(use_sigmoid=cfg["sigmoid"], norm_expert_weight=cfg["norm"], n_group=cfg["n_group"], topk_group=cfg["topk_group"])
+        with torch.no_grad():
+            for name, fn in (
+                ("fused", lambda: forward_gate_router(x, wg, K, fp32_output=True, **rk)),
+                ("two_step", lambda: forward_router(torch.matmul(x.float(), wg.t().float()), K, **rk)),
+            ):
+                for _ in range(3):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(20):
+                    fn()
+                torch.cuda.synchronize()
+                gate_us[name] = (time.perf_counter() - t0) / 20 * 1e6
+
     def bw(names, nbytes):
         t = next((timing[n] for n in names.split("|") if n in timing and timing[n]["calls"]), None)
         if t is None:
@@ -397,6 +419,7 @@ def main():
         "route_plan_us": timing.get("stm_route_plan", {}).get("avg_us"),
         "router_fwd_us": timing.get("stm_router_fwd", {}).get("avg_us"),
         "router_bwd_us": timing.get("stm_router_bwd", {}).get("avg_us"),
+        "gate_plus_router_fwd_us": gate_us or None,
         "swiglu_fwd_us": timing.get("stm_swiglu_fwd", {}).get("avg_us"),
         "swiglu_bwd_us": timing.get("stm_swiglu_bwd", {}).get("avg_us"),
     }

@@ -363,6 +363,26 @@ int stm_router_bwd(const void* logits, int logits_dtype, int64_t n_tokens, int n
                    int norm_weights, float eps, const int64_t* ids, const float* grad_weights,
                    const float* grad_aux_or_null, const int32_t* hist, void* grad_logits, stm_stream_t stream);
 
+/* The same with the gate GEMM in front (MoEGate / MoEGateFunction, moe_block.py:97-113 and
+ * moe_utils.py:64-82: logits = x @ gate_w^T): x [T, hidden] and gate_w [E, hidden] in bf16 or fp16,
+ * fp32 accumulation; the logits live in LDS only.  fp32_logits = 0 rounds them to the element type
+ * first, as a 16-bit gate output would be (fp32_output = False); 1 keeps them in fp32
+ * (fp32_output = True).  STM_ERR_UNSUPPORTED for fp32 inputs, hidden not a multiple of 16 or more
+ * than 512 experts: callers then compute the logits themselves and call stm_router_fwd.
+ * Workspace as for stm_router_fwd.
+ * stm_router_gate_bwd recomputes the logits the same way and writes d logits [T, E] (grad_dtype:
+ * the reference hands the gate's backward its gradient in x's type, moe_utils.py:75-82); d x and
+ * d gate_w are the two dense products of that matrix with gate_w and x. */
+int stm_router_gate_fwd(const void* x, const void* gate_w, int dtype, int hidden, int fp32_logits,
+                        const float* bias_or_null, int64_t n_tokens, int n_experts, int top_k, int use_sigmoid,
+                        int norm_weights, float eps, int n_group, int topk_group, int64_t* ids_out, float* weights_out,
+                        float* aux_out, int32_t* hist_out, float* me_out, void* workspace, size_t workspace_bytes,
+                        stm_stream_t stream);
+int stm_router_gate_bwd(const void* x, const void* gate_w, int dtype, int hidden, int fp32_logits, int64_t n_tokens,
+                        int n_experts, int top_k, int use_sigmoid, int norm_weights, float eps, const int64_t* ids,
+                        const float* grad_weights, const float* grad_aux_or_null, const int32_t* hist,
+                        void* grad_logits, int grad_dtype, stm_stream_t stream);
+
 /* Aux-loss-free load balancing, one MoE layer: bias[e] += sign(mean(tokens) - tokens[e]) * rate
  * (fp32 bias; sign(0) = 0), then tokens[e] = 0 if zero_tokens
  * (MoEBlock.update_router_balance_bias_per_gbs, moe_block.py:442-491, after its all-reduces). */

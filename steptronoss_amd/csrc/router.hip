@@ -75,16 +75,157 @@ __device__ __forceinline__ void token_scores(const RouterArgs& a, int64_t t, int
   }
 }
 
+// One token: scores from the logits of row t_in, selection, weights of row t_out; the column
+// sums and pick counts of this lane's experts are added to col / cnt.
+template <int V>
+__device__ __forceinline__ void route_one(const RouterArgs& a, int64_t t_in, int64_t t_out, int lane,
+                                          int64_t* __restrict__ ids, float* __restrict__ weights, float (&col)[V],
+                                          int32_t (&cnt)[V]) {
+  const int E = a.n_experts, K = a.top_k;
+  const int per_group = a.n_group > 1 ? E / a.n_group : E;
+  float p[V], c[V];
+  token_scores<V>(a, t_in, lane, p);
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    const int e = j * kWave + lane;
+    c[j] = e < E ? (a.bias ? p[j] + a.bias[e] : p[j]) : -INFINITY;
+  }
+  // ---- group-limited routing: keep the topk_group groups with the largest top-2 sums
+  if (a.n_group > 1) {
+    uint64_t keep = 0;
+    float my_gscore = -INFINITY;  // lane g keeps the score of group g (n_group <= 64)
+    for (int g = 0; g < a.n_group; ++g) {
+      float best = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        const int e = j * kWave + lane;
+        if (e < E && e / per_group == g) best = fmaxf(best, c[j]);
+      }
+      const float top1 = wave_max(best);
+      int n_top = 0;
+      float second = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        const int e = j * kWave + lane;
+        if (e < E && e / per_group == g) {
+          if (c[j] == top1)
+            ++n_top;
+          else
+            second = fmaxf(second, c[j]);
+        }
+      }
+      n_top = wave_sum(n_top);
+      second = wave_max(second);
+      const float gscore = per_group >= 2 ? top1 + (n_top >= 2 ? top1 : second) : top1;
+      if (lane == g) my_gscore = gscore;
+    }
+    for (int r = 0; r < a.topk_group; ++r) {  // largest score first, equal scores: lower group
+      const bool free_group = lane < a.n_group && !((keep >> lane) & 1);
+      float best = free_group ? my_gscore : -INFINITY;
+      int pick = free_group ? lane : INT32_MAX;
+      wave_argmax(best, pick);
+      if (pick != INT32_MAX) keep |= 1ull << pick;
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const int e = j * kWave + lane;
+      if (e < E && !((keep >> (e / per_group)) & 1)) c[j] = -INFINITY;
+    }
+  }
+  // ---- K rounds of arg-max; `taken` marks this lane's experts already chosen
+  uint32_t taken = 0;
+  float tp_sum = 0.f;
+  float my_tp = 0.f;  // lane r keeps the score of the r-th pick (K <= 64)
+  int my_id = 0;
+  for (int r = 0; r < K; ++r) {
+    float bv = -INFINITY;
+    int bi = INT32_MAX;
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const int e = j * kWave + lane;
+      if (e < E && !((taken >> j) & 1) && (c[j] > bv || (c[j] == bv && e < bi))) {
+        bv = c[j];
+        bi = e;
+      }
+    }
+    // a lane with nothing left still offers (-inf, its smallest free id) so that rows whose
+    // remaining scores are all -inf keep the ascending-id order of a stable sort
+    if (bi == INT32_MAX) {
+#pragma unroll
+      for (int j = V - 1; j >= 0; --j) {
+        const int e = j * kWave + lane;
+        if (e < E && !((taken >> j) & 1)) bi = e;
+      }
+    }
+    wave_argmax(bv, bi);
+    const int owner = bi % kWave, slot = bi / kWave;
+    float pv = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+      if (j == slot) pv = p[j];
+    pv = __shfl(pv, owner, kWave);
+    if (lane == owner) {
+      taken |= 1u << slot;
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        if (j == slot) ++cnt[j];
+    }
+    tp_sum += pv;
+    if (lane == r) {
+      my_tp = pv;
+      my_id = bi;
+    }
+  }
+  // ---- weights and score normalisation
+  float row_sum = 0.f;
+  if (a.use_sigmoid) {
+#pragma unroll
+    for (int j = 0; j < V; ++j) row_sum += p[j];
+    row_sum = wave_sum(row_sum) + a.eps;
+  }
+  const bool renorm = a.use_sigmoid || a.norm_weights;
+  if (lane < K) {
+    ids[t_out * K + lane] = my_id;
+    weights[t_out * K + lane] = renorm ? my_tp / (tp_sum + a.eps) : my_tp;
+  }
+#pragma unroll
+  for (int j = 0; j < V; ++j) col[j] += a.use_sigmoid ? p[j] / row_sum : p[j];
+}
+
+// Column sums and counts of a workgroup's tokens -> its row of the partials.
+template <int V>
+__device__ __forceinline__ void write_partials(const float (&col)[V], const int32_t (&cnt)[V], float* lds_col,
+                                               int32_t* lds_cnt, int n_experts, float* __restrict__ col_partial,
+                                               int32_t* __restrict__ cnt_partial) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    lds_col[wave * (V * kWave) + j * kWave + lane] = col[j];
+    lds_cnt[wave * (V * kWave) + j * kWave + lane] = cnt[j];
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < n_experts; e += kRouterWaves * kWave) {
+    float sum = 0.f;
+    int32_t n = 0;
+#pragma unroll
+    for (int w = 0; w < kRouterWaves; ++w) {
+      sum += lds_col[w * (V * kWave) + e];
+      n += lds_cnt[w * (V * kWave) + e];
+    }
+    col_partial[int64_t(blockIdx.x) * n_experts + e] = sum;
+    cnt_partial[int64_t(blockIdx.x) * n_experts + e] = n;
+  }
+}
+
 template <int V>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_fwd_kernel(RouterArgs a, int64_t* __restrict__ ids,
                                                                          float* __restrict__ weights,
                                                                          float* __restrict__ col_partial,
                                                                          int32_t* __restrict__ cnt_partial) {
-  __shared__ float lds_col[kRouterWaves][V * kWave];
-  __shared__ int32_t lds_cnt[kRouterWaves][V * kWave];
+  __shared__ float lds_col[kRouterWaves * V * kWave];
+  __shared__ int32_t lds_cnt[kRouterWaves * V * kWave];
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
-  const int E = a.n_experts, K = a.top_k;
   float col[V];
   int32_t cnt[V];
 #pragma unroll
@@ -92,135 +233,9 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_fwd_kernel(RouterA
     col[j] = 0.f;
     cnt[j] = 0;
   }
-  const int per_group = a.n_group > 1 ? E / a.n_group : E;
-
-  for (int64_t t = int64_t(blockIdx.x) * kRouterWaves + wave; t < a.n_tokens; t += int64_t(gridDim.x) * kRouterWaves) {
-    float p[V], c[V];
-    token_scores<V>(a, t, lane, p);
-#pragma unroll
-    for (int j = 0; j < V; ++j) {
-      const int e = j * kWave + lane;
-      c[j] = e < E ? (a.bias ? p[j] + a.bias[e] : p[j]) : -INFINITY;
-    }
-    // ---- group-limited routing: keep the topk_group groups with the largest top-2 sums
-    if (a.n_group > 1) {
-      uint64_t keep = 0;
-      float my_gscore = -INFINITY;  // lane g keeps the score of group g (n_group <= 64)
-      for (int g = 0; g < a.n_group; ++g) {
-        float best = -INFINITY;
-#pragma unroll
-        for (int j = 0; j < V; ++j) {
-          const int e = j * kWave + lane;
-          if (e < E && e / per_group == g) best = fmaxf(best, c[j]);
-        }
-        const float top1 = wave_max(best);
-        int n_top = 0;
-        float second = -INFINITY;
-#pragma unroll
-        for (int j = 0; j < V; ++j) {
-          const int e = j * kWave + lane;
-          if (e < E && e / per_group == g) {
-            if (c[j] == top1)
-              ++n_top;
-            else
-              second = fmaxf(second, c[j]);
-          }
-        }
-        n_top = wave_sum(n_top);
-        second = wave_max(second);
-        const float gscore = per_group >= 2 ? top1 + (n_top >= 2 ? top1 : second) : top1;
-        if (lane == g) my_gscore = gscore;
-      }
-      for (int r = 0; r < a.topk_group; ++r) {  // largest score first, equal scores: lower group
-        const bool free_group = lane < a.n_group && !((keep >> lane) & 1);
-        float best = free_group ? my_gscore : -INFINITY;
-        int pick = free_group ? lane : INT32_MAX;
-        wave_argmax(best, pick);
-        if (pick != INT32_MAX) keep |= 1ull << pick;
-      }
-#pragma unroll
-      for (int j = 0; j < V; ++j) {
-        const int e = j * kWave + lane;
-        if (e < E && !((keep >> (e / per_group)) & 1)) c[j] = -INFINITY;
-      }
-    }
-    // ---- K rounds of arg-max; `taken` marks this lane's experts already chosen
-    uint32_t taken = 0;
-    float tp_sum = 0.f;
-    float my_tp = 0.f;  // lane r keeps the score of the r-th pick (K <= 64)
-    int my_id = 0;
-    for (int r = 0; r < K; ++r) {
-      float bv = -INFINITY;
-      int bi = INT32_MAX;
-#pragma unroll
-      for (int j = 0; j < V; ++j) {
-        const int e = j * kWave + lane;
-        if (e < E && !((taken >> j) & 1) && (c[j] > bv || (c[j] == bv && e < bi))) {
-          bv = c[j];
-          bi = e;
-        }
-      }
-      // a lane with nothing left still offers (-inf, its smallest free id) so that rows whose
-      // remaining scores are all -inf keep the ascending-id order of a stable sort
-      if (bi == INT32_MAX) {
-#pragma unroll
-        for (int j = V - 1; j >= 0; --j) {
-          const int e = j * kWave + lane;
-          if (e < E && !((taken >> j) & 1)) bi = e;
-        }
-      }
-      wave_argmax(bv, bi);
-      const int owner = bi % kWave, slot = bi / kWave;
-      float pv = 0.f;
-#pragma unroll
-      for (int j = 0; j < V; ++j)
-        if (j == slot) pv = p[j];
-      pv = __shfl(pv, owner, kWave);
-      if (lane == owner) {
-        taken |= 1u << slot;
-#pragma unroll
-        for (int j = 0; j < V; ++j)
-          if (j == slot) ++cnt[j];
-      }
-      tp_sum += pv;
-      if (lane == r) {
-        my_tp = pv;
-        my_id = bi;
-      }
-    }
-    // ---- weights and score normalisation
-    float row_sum = 0.f;
-    if (a.use_sigmoid) {
-#pragma unroll
-      for (int j = 0; j < V; ++j) row_sum += p[j];
-      row_sum = wave_sum(row_sum) + a.eps;
-    }
-    const bool renorm = a.use_sigmoid || a.norm_weights;
-    if (lane < K) {
-      ids[t * K + lane] = my_id;
-      weights[t * K + lane] = renorm ? my_tp / (tp_sum + a.eps) : my_tp;
-    }
-#pragma unroll
-    for (int j = 0; j < V; ++j) col[j] += a.use_sigmoid ? p[j] / row_sum : p[j];
-  }
-  // ---- per-workgroup partials of the column sums and counts
-#pragma unroll
-  for (int j = 0; j < V; ++j) {
-    lds_col[wave][j * kWave + lane] = col[j];
-    lds_cnt[wave][j * kWave + lane] = cnt[j];
-  }
-  __syncthreads();
-  for (int e = threadIdx.x; e < E; e += kRouterWaves * kWave) {
-    float s = 0.f;
-    int32_t n = 0;
-#pragma unroll
-    for (int w = 0; w < kRouterWaves; ++w) {
-      s += lds_col[w][e];
-      n += lds_cnt[w][e];
-    }
-    col_partial[int64_t(blockIdx.x) * E + e] = s;
-    cnt_partial[int64_t(blockIdx.x) * E + e] = n;
-  }
+  for (int64_t t = int64_t(blockIdx.x) * kRouterWaves + wave; t < a.n_tokens; t += int64_t(gridDim.x) * kRouterWaves)
+    route_one<V>(a, t, t, lane, ids, weights, col, cnt);
+  write_partials<V>(col, cnt, lds_col, lds_cnt, a.n_experts, col_partial, cnt_partial);
 }
 
 // me[e] = sum_t score[t,e] / T, hist[e] = count, aux = E * sum_e me[e] * hist[e].
@@ -274,6 +289,94 @@ __global__ __launch_bounds__(1024) void router_finish_kernel(const float* __rest
   }
 }
 
+// d logits of one token (row t_out of ids / grad_w / grad_logits) from the logits of row t_in.
+template <int V>
+__device__ __forceinline__ void route_one_bwd(const RouterArgs& a, int64_t t_in, int64_t t_out, int lane,
+                                              const int64_t* __restrict__ ids, const float* __restrict__ grad_w,
+                                              const float (&dcol)[V], void* __restrict__ grad_logits, int grad_dtype) {
+  const int E = a.n_experts, K = a.top_k;
+  float p[V], dp[V];
+  token_scores<V>(a, t_in, lane, p);
+  // lane r < K holds the r-th pick
+  int my_id = -1;
+  float my_gw = 0.f, my_tp = 0.f;
+  if (lane < K) {
+    my_id = int(ids[t_out * K + lane]);
+    my_gw = grad_w[t_out * K + lane];
+  }
+  // fetch the picked scores from their owner lanes
+  for (int r = 0; r < K; ++r) {
+    const int e = __shfl(my_id, r, kWave);
+    float pv = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+      if (j == e / kWave) pv = p[j];
+    pv = __shfl(pv, e % kWave, kWave);
+    if (lane == r) my_tp = pv;
+  }
+  const bool renorm = a.use_sigmoid || a.norm_weights;
+  float dtp = my_gw;  // d L / d (picked raw score), lane r
+  if (renorm) {
+    const float s = wave_sum(lane < K ? my_tp : 0.f) + a.eps;
+    const float dot = wave_sum(lane < K ? my_gw * (my_tp / s) : 0.f);
+    dtp = (my_gw - dot) / s;
+  }
+  // d L / d raw score
+  if (a.use_sigmoid) {
+    float row_sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; ++j) row_sum += p[j];
+    row_sum = wave_sum(row_sum) + a.eps;
+    float dot = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; ++j) dot += dcol[j] * (p[j] / row_sum);
+    dot = wave_sum(dot);
+#pragma unroll
+    for (int j = 0; j < V; ++j) dp[j] = (dcol[j] - dot) / row_sum;
+  } else {
+#pragma unroll
+    for (int j = 0; j < V; ++j) dp[j] = dcol[j];
+  }
+  for (int r = 0; r < K; ++r) {
+    const int e = __shfl(my_id, r, kWave);
+    const float g = __shfl(dtp, r, kWave);
+    if (lane == e % kWave) {
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        if (j == e / kWave) dp[j] += g;
+    }
+  }
+  // through the activation
+  if (a.use_sigmoid) {
+#pragma unroll
+    for (int j = 0; j < V; ++j) dp[j] = dp[j] * p[j] * (1.f - p[j]);
+  } else {
+    float dot = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; ++j) dot += dp[j] * p[j];
+    dot = wave_sum(dot);
+#pragma unroll
+    for (int j = 0; j < V; ++j) dp[j] = p[j] * (dp[j] - dot);
+  }
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    const int e = j * kWave + lane;
+    if (e < E) store_logit(grad_logits, grad_dtype, t_out * E + e, dp[j]);
+  }
+}
+
+// d aux / d (normalised score) of this lane's experts
+template <int V>
+__device__ __forceinline__ void aux_column_grads(const RouterArgs& a, const float* grad_aux, const int32_t* hist, int lane,
+                                                 float (&dcol)[V]) {
+  const float gaux = grad_aux ? grad_aux[0] : 0.f;
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    const int e = j * kWave + lane;
+    dcol[j] = (e < a.n_experts && a.n_tokens > 0) ? gaux * float(a.n_experts) * float(hist[e]) / float(a.n_tokens) : 0.f;
+  }
+}
+
 // d logits from d weights and d aux.
 template <int V>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_bwd_kernel(RouterArgs a, const int64_t* __restrict__ ids,
@@ -283,84 +386,180 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_bwd_kernel(RouterA
                                                                          void* __restrict__ grad_logits) {
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
-  const int E = a.n_experts, K = a.top_k;
-  const float gaux = grad_aux ? grad_aux[0] : 0.f;
-  float dcol[V];  // d aux / d (normalised score) of this lane's experts
+  float dcol[V];
+  aux_column_grads<V>(a, grad_aux, hist, lane, dcol);
+  for (int64_t t = int64_t(blockIdx.x) * kRouterWaves + wave; t < a.n_tokens; t += int64_t(gridDim.x) * kRouterWaves)
+    route_one_bwd<V>(a, t, t, lane, ids, grad_w, dcol, grad_logits, a.logits_dtype);
+}
+
+// ---------------------------------------------------------------- gate GEMM in front of the router
+// logits = x * Wg^T (x [T, H], Wg [E, H], 16-bit elements, fp32 accumulation) computed per chunk of
+// 32 tokens into LDS and routed from there: the logits never reach HBM.  A workgroup's 16 waves
+// split a chunk's [32, E] tile into 32-expert blocks and, when there are fewer than 16 of those,
+// into ranges of the contraction as well; the partial tiles are added in a fixed order, so the
+// logits do not depend on the launch geometry.
+struct GateArgs {
+  const void* x;
+  const void* w;
+  int hidden;
+  int fp32_logits;  // 0: the logits are rounded to the element type first (a 16-bit gate output)
+};
+
+constexpr int kGateTokens = 32;
+constexpr int kGateStageFloats = kRouterWaves * 32 * 32;  // 16 partial 32 x 32 tiles
+
+typedef float gate_f32x16_t __attribute__((ext_vector_type(16)));
+typedef __bf16 gate_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 gate_f16x8_t __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ gate_f32x16_t gate_mfma(bf16_t, uint4 a, uint4 b, gate_f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(gate_bf16x8_t, a), __builtin_bit_cast(gate_bf16x8_t, b), c,
+                                                 0, 0, 0);
+}
+__device__ __forceinline__ gate_f32x16_t gate_mfma(f16_t, uint4 a, uint4 b, gate_f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(gate_f16x8_t, a), __builtin_bit_cast(gate_f16x8_t, b), c, 0,
+                                                0, 0);
+}
+
+// stage[tt * E + e] = logits of token t0 + tt (tt < 32) for every expert e; all threads take part.
+template <typename T>
+__device__ __forceinline__ void gate_tile(const GateArgs& g, int64_t t0, int64_t n_tokens, int E, float* stage) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int n_eb = (E + 31) / 32;         // 32-expert blocks (<= 16)
+  const int parts = kRouterWaves / n_eb;  // ranges of the contraction
+  const int eb = wave % n_eb, part = wave / n_eb;
+  if (part < parts) {
+    const int steps = g.hidden / 16;
+    const int per = (steps + parts - 1) / parts;
+    const int s0 = part * per, s1 = s0 + per < steps ? s0 + per : steps;
+    const int row = lane % 32, kc = (lane / 32) * 8;
+    const int64_t tok = t0 + row;
+    const int e = eb * 32 + row;
+    const bool live_a = tok < n_tokens, live_b = e < E;
+    const T* xa = static_cast<const T*>(g.x) + (live_a ? tok : 0) * g.hidden + kc;
+    const T* wb = static_cast<const T*>(g.w) + int64_t(live_b ? e : 0) * g.hidden + kc;
+    gate_f32x16_t acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+#pragma unroll 4
+    for (int st = s0; st < s1; ++st) {
+      const uint4 fa = live_a ? *reinterpret_cast<const uint4*>(xa + st * 16) : zero;
+      const uint4 fb = live_b ? *reinterpret_cast<const uint4*>(wb + st * 16) : zero;
+      acc = gate_mfma(T{}, fa, fb, acc);
+    }
+    // register 4*blk + q of lane l: token 8*blk + (l/32)*4 + q, expert eb*32 + l%32
+    float* tile = stage + part * (kGateTokens * E);
+    if (live_b) {
+#pragma unroll
+      for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) tile[(8 * blk + (lane / 32) * 4 + q) * E + e] = acc[blk * 4 + q];
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < kGateTokens * E; i += kRouterWaves * kWave) {
+    float v = stage[i];
+    for (int q = 1; q < parts; ++q) v += stage[q * (kGateTokens * E) + i];
+    stage[i] = g.fp32_logits ? v : to_float(from_float<T>(v));
+  }
+  __syncthreads();
+}
+
+template <int V, typename T>
+__global__ __launch_bounds__(kRouterWaves* kWave) void router_gate_fwd_kernel(RouterArgs a, GateArgs g,
+                                                                              int64_t* __restrict__ ids,
+                                                                              float* __restrict__ weights,
+                                                                              float* __restrict__ col_partial,
+                                                                              int32_t* __restrict__ cnt_partial) {
+  extern __shared__ __align__(16) unsigned char gate_smem[];
+  float* stage = reinterpret_cast<float*>(gate_smem);
+  float* lds_col = stage + kGateStageFloats;
+  int32_t* lds_cnt = reinterpret_cast<int32_t*>(lds_col + kRouterWaves * V * kWave);
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  float col[V];
+  int32_t cnt[V];
 #pragma unroll
   for (int j = 0; j < V; ++j) {
-    const int e = j * kWave + lane;
-    dcol[j] = (e < E && a.n_tokens > 0) ? gaux * float(E) * float(hist[e]) / float(a.n_tokens) : 0.f;
+    col[j] = 0.f;
+    cnt[j] = 0;
   }
-  for (int64_t t = int64_t(blockIdx.x) * kRouterWaves + wave; t < a.n_tokens; t += int64_t(gridDim.x) * kRouterWaves) {
-    float p[V], dp[V];
-    token_scores<V>(a, t, lane, p);
-    // lane r < K holds the r-th pick
-    int my_id = -1;
-    float my_gw = 0.f, my_tp = 0.f;
-    if (lane < K) {
-      my_id = int(ids[t * K + lane]);
-      my_gw = grad_w[t * K + lane];
-    }
-    // fetch the picked scores from their owner lanes
-    for (int r = 0; r < K; ++r) {
-      const int e = __shfl(my_id, r, kWave);
-      float pv = 0.f;
-#pragma unroll
-      for (int j = 0; j < V; ++j)
-        if (j == e / kWave) pv = p[j];
-      pv = __shfl(pv, e % kWave, kWave);
-      if (lane == r) my_tp = pv;
-    }
-    const bool renorm = a.use_sigmoid || a.norm_weights;
-    float dtp = my_gw;  // d L / d (picked raw score), lane r
-    if (renorm) {
-      const float s = wave_sum(lane < K ? my_tp : 0.f) + a.eps;
-      const float dot = wave_sum(lane < K ? my_gw * (my_tp / s) : 0.f);
-      dtp = (my_gw - dot) / s;
-    }
-    // d L / d raw score
-    if (a.use_sigmoid) {
-      float row_sum = 0.f;
-#pragma unroll
-      for (int j = 0; j < V; ++j) row_sum += p[j];
-      row_sum = wave_sum(row_sum) + a.eps;
-      float dot = 0.f;
-#pragma unroll
-      for (int j = 0; j < V; ++j) dot += dcol[j] * (p[j] / row_sum);
-      dot = wave_sum(dot);
-#pragma unroll
-      for (int j = 0; j < V; ++j) dp[j] = (dcol[j] - dot) / row_sum;
-    } else {
-#pragma unroll
-      for (int j = 0; j < V; ++j) dp[j] = dcol[j];
-    }
-    for (int r = 0; r < K; ++r) {
-      const int e = __shfl(my_id, r, kWave);
-      const float g = __shfl(dtp, r, kWave);
-      if (lane == e % kWave) {
-#pragma unroll
-        for (int j = 0; j < V; ++j)
-          if (j == e / kWave) dp[j] += g;
-      }
-    }
-    // through the activation
-    if (a.use_sigmoid) {
-#pragma unroll
-      for (int j = 0; j < V; ++j) dp[j] = dp[j] * p[j] * (1.f - p[j]);
-    } else {
-      float dot = 0.f;
-#pragma unroll
-      for (int j = 0; j < V; ++j) dot += dp[j] * p[j];
-      dot = wave_sum(dot);
-#pragma unroll
-      for (int j = 0; j < V; ++j) dp[j] = p[j] * (dp[j] - dot);
-    }
-#pragma unroll
-    for (int j = 0; j < V; ++j) {
-      const int e = j * kWave + lane;
-      if (e < E) store_logit(grad_logits, a.logits_dtype, t * E + e, dp[j]);
-    }
+  RouterArgs staged = a;  // the router reads this chunk's logits from LDS, as fp32
+  staged.logits = stage;
+  staged.logits_dtype = STM_F32;
+  for (int64_t t0 = int64_t(blockIdx.x) * kGateTokens; t0 < a.n_tokens; t0 += int64_t(gridDim.x) * kGateTokens) {
+    gate_tile<T>(g, t0, a.n_tokens, a.n_experts, stage);
+    for (int tt = wave; tt < kGateTokens; tt += kRouterWaves)
+      if (t0 + tt < a.n_tokens) route_one<V>(staged, tt, t0 + tt, lane, ids, weights, col, cnt);
+    __syncthreads();  // the next chunk overwrites the stage
   }
+  write_partials<V>(col, cnt, lds_col, lds_cnt, a.n_experts, col_partial, cnt_partial);
+}
+
+template <int V, typename T>
+__global__ __launch_bounds__(kRouterWaves* kWave) void router_gate_bwd_kernel(RouterArgs a, GateArgs g,
+                                                                              const int64_t* __restrict__ ids,
+                                                                              const float* __restrict__ grad_w,
+                                                                              const float* __restrict__ grad_aux,
+                                                                              const int32_t* __restrict__ hist,
+                                                                              void* __restrict__ grad_logits,
+                                                                              int grad_dtype) {
+  extern __shared__ __align__(16) unsigned char gate_smem[];
+  float* stage = reinterpret_cast<float*>(gate_smem);
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  float dcol[V];
+  aux_column_grads<V>(a, grad_aux, hist, lane, dcol);
+  RouterArgs staged = a;
+  staged.logits = stage;
+  staged.logits_dtype = STM_F32;
+  for (int64_t t0 = int64_t(blockIdx.x) * kGateTokens; t0 < a.n_tokens; t0 += int64_t(gridDim.x) * kGateTokens) {
+    gate_tile<T>(g, t0, a.n_tokens, a.n_experts, stage);
+    for (int tt = wave; tt < kGateTokens; tt += kRouterWaves)
+      if (t0 + tt < a.n_tokens) route_one_bwd<V>(staged, tt, t0 + tt, lane, ids, grad_w, dcol, grad_logits, grad_dtype);
+    __syncthreads();
+  }
+}
+
+inline int gate_blocks(int64_t n_tokens) {
+  const int64_t want = (n_tokens + kGateTokens - 1) / kGateTokens;
+  return int(want < 1 ? 1 : (want > 512 ? 512 : want));
+}
+
+// shapes the fused gate takes: 16-bit elements, hidden a multiple of 16, at most 512 experts
+inline int check_gate_args(const void* x, const void* w, int dtype, int hidden, int n_experts) {
+  if (dtype != STM_BF16 && dtype != STM_F16) return STM_ERR_UNSUPPORTED;
+  if (hidden <= 0 || hidden % 16 != 0 || n_experts > 32 * kRouterWaves) return STM_ERR_UNSUPPORTED;
+  if (!aligned_to(x, 16) || !aligned_to(w, 16)) return STM_ERR_UNSUPPORTED;
+  return STM_OK;
+}
+
+template <typename K>
+int allow_large_lds(K kernel, size_t bytes) {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                             int(bytes)) == hipSuccess
+             ? STM_OK
+             : STM_ERR_LAUNCH;
+}
+
+template <int V, typename T>
+int launch_gate_fwd(const RouterArgs& a, const GateArgs& g, int blocks, int64_t* ids, float* weights, float* col_partial,
+                    int32_t* cnt_partial, hipStream_t s) {
+  const size_t lds = size_t(kGateStageFloats) * 4 + size_t(kRouterWaves) * V * kWave * 8;
+  if (allow_large_lds(router_gate_fwd_kernel<V, T>, lds) != STM_OK) return STM_ERR_LAUNCH;
+  router_gate_fwd_kernel<V, T><<<blocks, kRouterWaves * kWave, lds, s>>>(a, g, ids, weights, col_partial, cnt_partial);
+  return STM_OK;
+}
+
+template <int V, typename T>
+int launch_gate_bwd(const RouterArgs& a, const GateArgs& g, int blocks, const int64_t* ids, const float* grad_w,
+                    const float* grad_aux, const int32_t* hist, void* grad_logits, int grad_dtype, hipStream_t s) {
+  const size_t lds = size_t(kGateStageFloats) * 4;
+  if (allow_large_lds(router_gate_bwd_kernel<V, T>, lds) != STM_OK) return STM_ERR_LAUNCH;
+  router_gate_bwd_kernel<V, T><<<blocks, kRouterWaves * kWave, lds, s>>>(a, g, ids, grad_w, grad_aux, hist, grad_logits,
+                                                                         grad_dtype);
+  return STM_OK;
 }
 
 // Aux-loss-free load balancing: bias[e] += sign(mean(tokens) - tokens[e]) * rate, then the token
@@ -462,6 +661,65 @@ int stm_router_bwd(const void* logits, int logits_dtype, int64_t n_tokens, int n
   const int need = (n_experts + kWave - 1) / kWave;
   STM_ROUTER_DISPATCH(need, (router_bwd_kernel<V><<<blocks, kRouterWaves * kWave, 0, s>>>(
                                 a, ids, grad_weights, grad_aux_or_null, hist, grad_logits)));
+  return launch_status();
+}
+
+int stm_router_gate_fwd(const void* x, const void* gate_w, int dtype, int hidden, int fp32_logits,
+                        const float* bias_or_null, int64_t n_tokens, int n_experts, int top_k, int use_sigmoid,
+                        int norm_weights, float eps, int n_group, int topk_group, int64_t* ids_out, float* weights_out,
+                        float* aux_out, int32_t* hist_out, float* me_out, void* workspace, size_t workspace_bytes,
+                        stm_stream_t stream) {
+  using namespace stm;
+  RouterArgs a{nullptr, STM_F32, bias_or_null, n_tokens, n_experts, top_k, use_sigmoid, norm_weights,
+               n_group, topk_group,   eps};
+  int st = check_router_args(a);
+  if (st != STM_OK) return st;
+  if (n_tokens > 0 && n_experts > 0 && (!x || !gate_w)) return STM_ERR_ARG;
+  st = check_gate_args(x, gate_w, dtype, hidden, n_experts);
+  if (st != STM_OK) return st;
+  if (!aux_out || (n_experts > 0 && (!hist_out || !me_out))) return STM_ERR_ARG;
+  if (n_tokens > 0 && top_k > 0 && (!ids_out || !weights_out)) return STM_ERR_ARG;
+  if (workspace_bytes < stm_router_workspace_bytes(n_tokens, n_experts) || !workspace) return STM_ERR_WORKSPACE;
+  hipStream_t s = as_stream(stream);
+  const int blocks = gate_blocks(n_tokens);  // never more than router_blocks(): the workspace holds the partial rows
+  float* col_partial = static_cast<float*>(workspace);
+  int32_t* cnt_partial = reinterpret_cast<int32_t*>(col_partial + size_t(blocks) * n_experts);
+  GateArgs g{x, gate_w, hidden, fp32_logits};
+  const int need = (n_experts + kWave - 1) / kWave;
+  if (dtype == STM_BF16) {
+    STM_ROUTER_DISPATCH(need, (st = launch_gate_fwd<V, bf16_t>(a, g, blocks, ids_out, weights_out, col_partial, cnt_partial, s)));
+  } else {
+    STM_ROUTER_DISPATCH(need, (st = launch_gate_fwd<V, f16_t>(a, g, blocks, ids_out, weights_out, col_partial, cnt_partial, s)));
+  }
+  if (st != STM_OK) return st;
+  router_finish_kernel<<<1, 1024, 0, s>>>(col_partial, cnt_partial, blocks, n_experts, n_tokens, me_out, hist_out,
+                                          aux_out);
+  return launch_status();
+}
+
+int stm_router_gate_bwd(const void* x, const void* gate_w, int dtype, int hidden, int fp32_logits, int64_t n_tokens,
+                        int n_experts, int top_k, int use_sigmoid, int norm_weights, float eps, const int64_t* ids,
+                        const float* grad_weights, const float* grad_aux_or_null, const int32_t* hist,
+                        void* grad_logits, int grad_dtype, stm_stream_t stream) {
+  using namespace stm;
+  RouterArgs a{nullptr, STM_F32, nullptr, n_tokens, n_experts, top_k, use_sigmoid, norm_weights, 1, 1, eps};
+  int st = check_router_args(a);
+  if (st != STM_OK) return st;
+  if (grad_dtype < STM_F32 || grad_dtype > STM_BF16) return STM_ERR_UNSUPPORTED;
+  if (n_tokens == 0 || n_experts == 0) return STM_OK;
+  if (!x || !gate_w || !grad_logits || !hist || (top_k > 0 && (!ids || !grad_weights))) return STM_ERR_ARG;
+  st = check_gate_args(x, gate_w, dtype, hidden, n_experts);
+  if (st != STM_OK) return st;
+  hipStream_t s = as_stream(stream);
+  const int blocks = gate_blocks(n_tokens);
+  GateArgs g{x, gate_w, hidden, fp32_logits};
+  const int need = (n_experts + kWave - 1) / kWave;
+  if (dtype == STM_BF16) {
+    STM_ROUTER_DISPATCH(need, (st = launch_gate_bwd<V, bf16_t>(a, g, blocks, ids, grad_weights, grad_aux_or_null, hist, grad_logits, grad_dtype, s)));
+  } else {
+    STM_ROUTER_DISPATCH(need, (st = launch_gate_bwd<V, f16_t>(a, g, blocks, ids, grad_weights, grad_aux_or_null, hist, grad_logits, grad_dtype, s)));
+  }
+  if (st != STM_OK) return st;
   return launch_status();
 }
 

@@ -16,7 +16,7 @@ from torch import nn
 from steptronoss_amd import _lib
 from steptronoss_amd._lib import call, dtype_code, ptr, require_gpu, stream
 from steptronoss_amd.model.common.feed_forward import swiglu
-from steptronoss_amd.model.utils.moe_utils import routed_grouped_ffn
+from steptronoss_amd.model.utils.moe_utils import routed_grouped_ffn, settings
 
 
 class _Router(torch.autograd.Function):
@@ -92,6 +92,95 @@ def forward_router(
     return _Router.apply(logits, balance_bias, top_k, use_sigmoid, norm_expert_weight, eps, n_group, topk_group)
 
 
+class _GateRouter(torch.autograd.Function):
+    """Gate GEMM and router in one kernel: ``forward_router(x @ gate_w^T)`` with the logits kept in
+    LDS.  The backward recomputes them the same way, writes ``d logits`` in ``x``'s dtype (the
+    reference's ``MoEGateFunction.backward`` casts to it, moe_utils.py:75-82) and forms
+    ``d x = d logits @ gate_w`` and ``d gate_w = d logits^T @ x`` as two dense library GEMMs."""
+
+    @staticmethod
+    def forward(ctx, x, gate_w, bias, top_k, use_sigmoid, norm_weights, eps, n_group, topk_group, fp32_logits):
+        dev = require_gpu(x, gate_w, bias)
+        xc, wc = x.contiguous(), gate_w.contiguous()
+        T, H = xc.shape
+        E = wc.shape[0]
+        ids = torch.empty((T, top_k), device=dev, dtype=torch.int64)
+        weights = torch.empty((T, top_k), device=dev, dtype=torch.float32)
+        aux = torch.empty((), device=dev, dtype=torch.float32)
+        hist = torch.empty((E,), device=dev, dtype=torch.int32)
+        me = torch.empty((E,), device=dev, dtype=torch.float32)
+        with torch.cuda.device(dev):
+            nbytes = _lib.load().stm_router_workspace_bytes(T, E)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            b = None if bias is None else bias.to(torch.float32).contiguous()
+            call(
+                "stm_router_gate_fwd", ptr(xc), ptr(wc), dtype_code(xc.dtype), H, int(fp32_logits), ptr(b), T, E, top_k,
+                int(use_sigmoid), int(norm_weights), float(eps), int(n_group), int(topk_group), ptr(ids), ptr(weights),
+                ptr(aux), ptr(hist), ptr(me), ptr(ws), ws.numel(), stream(),
+            )  # fmt: skip
+        ctx.save_for_backward(xc, wc, ids, hist)
+        ctx.cfg = (top_k, use_sigmoid, norm_weights, eps, fp32_logits)
+        ctx.mark_non_differentiable(ids, hist)
+        return ids, weights, aux, hist
+
+    @staticmethod
+    def backward(ctx, _g_ids, g_weights, g_aux, _g_hist):
+        x, gate_w, ids, hist = ctx.saved_tensors
+        top_k, use_sigmoid, norm_weights, eps, fp32_logits = ctx.cfg
+        T, H = x.shape
+        E = gate_w.shape[0]
+        with torch.cuda.device(x.device):
+            gw = (
+                torch.zeros((T, top_k), device=x.device, dtype=torch.float32)
+                if g_weights is None
+                else g_weights.to(torch.float32).contiguous()
+            )
+            ga = None if g_aux is None else g_aux.to(torch.float32).reshape(1).contiguous()
+            gl = torch.empty((T, E), device=x.device, dtype=x.dtype)
+            call(
+                "stm_router_gate_bwd", ptr(x), ptr(gate_w), dtype_code(x.dtype), H, int(fp32_logits), T, E, top_k,
+                int(use_sigmoid), int(norm_weights), float(eps), ptr(ids), ptr(gw), ptr(ga), ptr(hist), ptr(gl),
+                dtype_code(gl.dtype), stream(),
+            )  # fmt: skip
+            gx = torch.matmul(gl, gate_w) if ctx.needs_input_grad[0] else None
+            gwt = torch.matmul(gl.t(), x) if ctx.needs_input_grad[1] else None
+        return gx, gwt, None, None, None, None, None, None, None, None
+
+
+def gate_router_takes(x: torch.Tensor, gate_w: torch.Tensor) -> bool:
+    """Shapes the fused gate + router kernel takes (others compute the logits first)."""
+    return (
+        x.is_cuda and x.dim() == 2 and x.dtype in (torch.bfloat16, torch.float16) and gate_w.dtype == x.dtype
+        and x.shape[1] % 16 == 0 and gate_w.shape[0] <= 512 and gate_w.shape[1] == x.shape[1]
+    )  # fmt: skip
+
+
+def forward_gate_router(
+    x: torch.Tensor,
+    gate_weight: torch.Tensor,
+    top_k: int,
+    *,
+    fp32_output: bool = False,
+    use_sigmoid: bool = False,
+    norm_expert_weight: bool = True,
+    balance_bias: torch.Tensor | None = None,
+    n_group: int = 1,
+    topk_group: int = 1,
+):
+    """``forward_router(MoEGate(x))`` (reference moe_block.py:97-113, 224-292) as one kernel: the
+    logits ``x @ gate_weight^T`` (fp32 accumulation; rounded to ``x``'s dtype unless ``fp32_output``)
+    are routed straight from LDS.  Same return values as :func:`forward_router`; differentiable
+    in ``x`` and ``gate_weight``."""
+    if top_k > gate_weight.shape[0]:
+        raise ValueError("top_k must not exceed the number of experts")
+    if not gate_router_takes(x, gate_weight):
+        raise ValueError("forward_gate_router: bf16/fp16 x [T, H] with H a multiple of 16 and at most 512 experts")
+    eps = 1e-20 if balance_bias is not None else 0.0
+    return _GateRouter.apply(
+        x, gate_weight, balance_bias, top_k, use_sigmoid, norm_expert_weight, eps, n_group, topk_group, fp32_output
+    )
+
+
 class _BindAuxLoss(torch.autograd.Function):
     """Identity on the output; hands ``aux_loss`` a gradient of one in backward (reference
     steptronoss/model/utils/utils.py:68-90)."""
@@ -113,7 +202,8 @@ def bind_aux_loss(output: torch.Tensor, aux_loss: torch.Tensor) -> torch.Tensor:
 
 class MoEGate(nn.Module):
     """``logits = x @ W^T`` (fp32 when ``fp32_output``); reference moe_block.py:97-113 and
-    moe_utils.py:64-82.  A plain dense GEMM next to the path, left to the BLAS library."""
+    moe_utils.py:64-82.  Called on its own it is a plain dense GEMM left to the BLAS library;
+    ``MoEBlock`` folds it into the router kernel (``forward_gate_router``) when it can."""
 
     def __init__(self, dim: int, num_experts: int, fp32_output: bool = False, device=None, dtype=None):
         super().__init__()
@@ -208,9 +298,16 @@ class MoEBlock(nn.Module):
         the sum of both, the scaling and the addition done by the combine kernel."""
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
-        if logits is None:
-            logits = self.gate(x2)
-        ids, weights, aux, hist = self.route(logits)
+        if logits is None and settings.fuse_gate and gate_router_takes(x2, self.gate.weight):
+            ids, weights, aux, hist = forward_gate_router(
+                x2, self.gate.weight, self.top_k, fp32_output=self.gate.fp32_output, use_sigmoid=self.use_sigmoid_router,
+                norm_expert_weight=self.norm_expert_weight, balance_bias=self.router_balance_bias, n_group=self.n_group,
+                topk_group=self.topk_group,
+            )  # fmt: skip
+        else:
+            if logits is None:
+                logits = self.gate(x2)
+            ids, weights, aux, hist = self.route(logits)
         if self.local_tokens_per_expert is not None and self.training:
             with torch.no_grad():  # reference moe_block.py:283-290
                 self.local_tokens_per_expert += hist.to(self.local_tokens_per_expert.dtype)

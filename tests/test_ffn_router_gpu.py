@@ -593,3 +593,111 @@ def test_shared_expert_layer_matches_the_unfused_composition():
     assert len(fused) == len(unfused)
     for a, b in zip(fused, unfused):
         assert rel_l2(a, b.float()) <= 1e-2  # same roundings except where autograd sums two gradient paths
+
+
+# ------------------------------------------------------------------ gate GEMM in front of the router
+def _grid(shape, gen, steps=16, scale=8.0):
+    """Values k / scale, |k| <= steps: products and sums of a few hundred of them are exact in fp32
+    in any order, so the gate's logits do not depend on how the GEMM adds them up."""
+    return torch.randint(-steps, steps + 1, shape, generator=gen).float() / scale
+
+
+GATE_CASES = [
+    # T, H, E, K, sigmoid, norm, bias, n_group, topk_group, fp32_output, dtype
+    (1000, 256, 128, 8, False, True, False, 1, 1, True, torch.bfloat16),
+    (1000, 256, 128, 8, False, True, False, 1, 1, False, torch.bfloat16),
+    (300, 512, 256, 8, True, True, True, 8, 4, True, torch.bfloat16),
+    (77, 64, 8, 2, False, False, False, 1, 1, False, torch.bfloat16),
+    (513, 128, 60, 6, False, True, True, 1, 1, True, torch.float16),
+    (64, 7168, 256, 8, True, True, False, 8, 4, True, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("T,H,E,K,sig,norm,bias,ng,tg,fp32_out,dtype", GATE_CASES)
+def test_gate_router_matches_oracle(T, H, E, K, sig, norm, bias, ng, tg, fp32_out, dtype):
+    # MoEGate + forward_router of the reference (moe_block.py:97-113, 224-292) as one kernel
+    gen = torch.Generator().manual_seed(13)
+    x = _grid((T, H), gen, steps=8 if H > 1024 else 16)
+    wg = _grid((E, H), gen, steps=8 if H > 1024 else 16)
+    bb = (torch.randn(E, generator=gen) * 0.01) if bias else None
+    kw = dict(use_sigmoid=sig, norm_expert_weight=norm, balance_bias=bb, n_group=ng, topk_group=tg)
+    xr, wr = x.clone().requires_grad_(True), wg.clone().requires_grad_(True)
+    logits = xr @ wr.t()
+    if not fp32_out:  # a 16-bit gate output: the exact sums rounded once (straight-through for the gradient)
+        logits = logits + (logits.detach().to(dtype).float() - logits.detach())
+    logits = logits * 0.125  # keeps the scores apart (applied to both sides through the weights below)
+    ref_ids, ref_w, ref_aux, ref_hist = O.forward_router(logits, K, **kw)
+    xg = x.to(dtype).to(DEV).requires_grad_(True)
+    wgd = (wg * 0.125).to(dtype).to(DEV).requires_grad_(True)  # exact: a power of two
+    ids, w, aux, hist = B.forward_gate_router(
+        xg, wgd, K, fp32_output=fp32_out, **{**kw, "balance_bias": None if bb is None else bb.to(DEV)}
+    )
+    if not fp32_out:
+        # the reference rounds x @ (w/8)^T, the oracle above rounded (x @ w^T) and then divided by 8: the same
+        # numbers, since a division by 8 commutes with the rounding
+        pass
+    assert torch.equal(ids.cpu(), ref_ids), f"{int((ids.cpu() != ref_ids).any(1).sum())} tokens differ"
+    assert torch.equal(hist.cpu(), ref_hist)
+    assert torch.allclose(w.cpu(), ref_w, rtol=2e-5, atol=1e-7)
+    assert torch.allclose(aux.cpu(), ref_aux, rtol=2e-5)
+    # the logits are the fused kernel's own: the two-step path gives the same picks
+    two_step = B.forward_router(
+        (xg.detach() @ wgd.detach().t()).float() if not fp32_out else xg.detach().float() @ wgd.detach().float().t(),
+        K, **{**kw, "balance_bias": None if bb is None else bb.to(DEV)},
+    )  # fmt: skip
+    assert torch.equal(two_step[0], ids)
+    # gradients: d logits goes through the element type (as the reference's gate backward casts it)
+    gw = torch.randn(T, K, generator=gen)
+    (w * gw.to(DEV)).sum().add(aux * 0.37).backward()
+    ((ref_w * gw).sum() + ref_aux * 0.37).backward()
+    assert rel_l2(xg.grad, xr.grad) <= 1e-2
+    assert rel_l2(wgd.grad, wr.grad * 8.0) <= 1e-2  # d (w / 8) = 8 d w
+
+
+@pytest.mark.parametrize("fuse_gate", [True, False])
+@pytest.mark.parametrize("fp32_gate", [True, False])
+def test_moe_block_with_its_own_gate(fuse_gate, fp32_gate):
+    # MoEBlock.forward without ready-made logits (reference moe_block.py:376-420): gate, router, experts
+    gen = torch.Generator().manual_seed(21)
+    T, H, E, K, Fh = 1024, 128, 16, 4, 64
+    x = _grid((T, H), gen)
+    wg = _grid((E, H), gen) * 0.125
+    w1 = (torch.randn(E, 2 * Fh, H, generator=gen) * 0.1).bfloat16()
+    w2 = (torch.randn(E, H, Fh, generator=gen) * 0.1).bfloat16()
+    go = torch.randn(T, H, generator=gen).bfloat16()
+    ref_in = [t.clone().float().requires_grad_(True) for t in (x, wg, w1, w2)]
+    logits = ref_in[0] @ ref_in[1].t()
+    if not fp32_gate:
+        logits = logits + (logits.detach().bfloat16().float() - logits.detach())
+    ref, ref_ids, _, _ = O.moe_layer(ref_in[0], logits, ref_in[2], ref_in[3], top_k=K, aux_loss_coef=0.01)
+    ref.backward(go.float())
+    blk = B.MoEBlock(H, Fh, E, K, aux_loss_coef=0.01, fp32_gate_output=fp32_gate, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        blk.gate.weight.copy_(wg)
+        blk.experts.w1.copy_(w1)
+        blk.experts.w2.copy_(w2)
+    xg = x.bfloat16().to(DEV).requires_grad_(True)
+    old = M.settings.fuse_gate
+    try:
+        M.settings.fuse_gate = fuse_gate
+        from steptronoss_amd.profiling import KernelTimer
+
+        with KernelTimer() as kt:
+            out = blk(xg)
+            out.backward(go.to(DEV))
+        assert ("stm_router_gate_fwd" in kt.summary()) == fuse_gate
+        assert ("stm_router_fwd" in kt.summary()) == (not fuse_gate)
+    finally:
+        M.settings.fuse_gate = old
+    ids = B.forward_router(logits.detach().to(DEV), K)[0]
+    assert torch.equal(ids.cpu(), ref_ids)
+    errs = {
+        "out": rel_l2(out, ref),
+        "dw1": rel_l2(blk.experts.w1.grad, ref_in[2].grad),
+        "dw2": rel_l2(blk.experts.w2.grad, ref_in[3].grad),
+    }
+    assert max(errs.values()) <= BF16_TOL, errs
+    # d x and d gate weight carry d logits, rounded to bf16 on its way into the two gate GEMMs and built
+    # from the combine-weight gradients (sums of bf16-rounded dot products): twice the bar
+    assert rel_l2(xg.grad, ref_in[0].grad) <= 2 * BF16_TOL
+    assert rel_l2(blk.gate.weight.grad, ref_in[1].grad) <= 5e-2
