@@ -60,7 +60,13 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(const T* __restrict__
   float v[8];
   const bool in = live && c0 < cols;
   if (in) {
-    const In8<T> raw = *reinterpret_cast<const In8<T>*>(x + r * cols + c0);
+    In8<T> raw;
+    if constexpr (sizeof(In8<T>) == 16) {  // streamed: every input byte is read once
+      typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+      raw = __builtin_bit_cast(In8<T>, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + r * cols + c0)));
+    } else {
+      raw = *reinterpret_cast<const In8<T>*>(x + r * cols + c0);
+    }
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = to_float(raw.v[e]);
   } else {
