@@ -138,32 +138,39 @@ __device__ __forceinline__ void route_one(const RouterArgs& a, int64_t t_in, int
   float my_tp = 0.f;  // lane r keeps the score of the r-th pick (K <= 64)
   int my_id = 0;
   for (int r = 0; r < K; ++r) {
+    // the largest remaining score, then its lowest expert id: ids grow with (j, lane), so the
+    // first j with a lane holding that score, and there the first such lane
     float bv = -INFINITY;
-    int bi = INT32_MAX;
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+      if (!((taken >> j) & 1)) bv = fmaxf(bv, c[j]);
+    const float top = wave_max(bv);
+    int slot = -1, owner = 0;
 #pragma unroll
     for (int j = 0; j < V; ++j) {
-      const int e = j * kWave + lane;
-      if (e < E && !((taken >> j) & 1) && (c[j] > bv || (c[j] == bv && e < bi))) {
-        bv = c[j];
-        bi = e;
+      const uint64_t holders = __ballot(j * kWave + lane < E && !((taken >> j) & 1) && c[j] == top);
+      if (slot < 0 && holders != 0) {
+        slot = j;
+        owner = __builtin_ctzll(holders);
       }
     }
-    // a lane with nothing left still offers (-inf, its smallest free id) so that rows whose
-    // remaining scores are all -inf keep the ascending-id order of a stable sort
-    if (bi == INT32_MAX) {
+    if (slot < 0) {  // nothing compares equal (NaN scores): the lowest id not taken yet
 #pragma unroll
-      for (int j = V - 1; j >= 0; --j) {
-        const int e = j * kWave + lane;
-        if (e < E && !((taken >> j) & 1)) bi = e;
+      for (int j = 0; j < V; ++j) {
+        const uint64_t free_lanes = __ballot(j * kWave + lane < E && !((taken >> j) & 1));
+        if (slot < 0 && free_lanes != 0) {
+          slot = j;
+          owner = __builtin_ctzll(free_lanes);
+        }
       }
+      if (slot < 0) slot = 0;  // (K > E is rejected by the caller)
     }
-    wave_argmax(bv, bi);
-    const int owner = bi % kWave, slot = bi / kWave;
+    const int bi = slot * kWave + owner;
     float pv = 0.f;
 #pragma unroll
     for (int j = 0; j < V; ++j)
       if (j == slot) pv = p[j];
-    pv = __shfl(pv, owner, kWave);
+    pv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pv), owner));
     if (lane == owner) {
       taken |= 1u << slot;
 #pragma unroll
@@ -394,10 +401,12 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_bwd_kernel(RouterA
 
 // ---------------------------------------------------------------- gate GEMM in front of the router
 // logits = x * Wg^T (x [T, H], Wg [E, H], 16-bit elements, fp32 accumulation) computed per chunk of
-// 32 tokens into LDS and routed from there: the logits never reach HBM.  A workgroup's 16 waves
-// split a chunk's [32, E] tile into 32-expert blocks and, when there are fewer than 16 of those,
-// into ranges of the contraction as well; the partial tiles are added in a fixed order, so the
-// logits do not depend on the launch geometry.
+// 64 tokens (32 when the logits of 64 would not fit) into LDS and routed from there: the logits
+// never reach HBM.  A workgroup's 16 waves split a chunk's [tokens, E] tile into blocks of 64
+// experts and, as there are fewer than 16 of those, into ranges of the contraction as well; the
+// partial tiles are added in a fixed order that depends on E and the hidden size alone, so the
+// forward pass and the recomputation in the backward pass see the same logits bit for bit,
+// whatever the launch geometry.
 struct GateArgs {
   const void* x;
   const void* w;
@@ -405,8 +414,39 @@ struct GateArgs {
   int fp32_logits;  // 0: the logits are rounded to the element type first (a 16-bit gate output)
 };
 
-constexpr int kGateTokens = 32;
-constexpr int kGateStageFloats = kRouterWaves * 32 * 32;  // 16 partial 32 x 32 tiles
+constexpr int kGateExpertBlocks = 2;           // 32-expert blocks of one wave's tile
+constexpr int kGateLdsBudget = 144 * 1024;     // stage + the forward kernel's partial rows
+constexpr int kGatePrefetch = 2;               // contraction steps in flight ahead of the matrix unit
+
+template <int V>
+struct GateShape {
+  static constexpr int kPartialBytes = kRouterWaves * V * kWave * 8;
+};
+
+// 32-token blocks of a chunk: two where the chunk's logits fit in LDS beside the partial rows
+inline int gate_token_blocks(int n_experts) {
+  const int lanes_per_row = (n_experts + kWave - 1) / kWave;
+  const int v = lanes_per_row <= 1 ? 1 : lanes_per_row <= 2 ? 2 : lanes_per_row <= 4 ? 4 : lanes_per_row <= 8 ? 8 : 16;
+  return 64 * n_experts * 4 + kRouterWaves * v * kWave * 8 <= kGateLdsBudget ? 2 : 1;
+}
+
+// how a chunk's work is split; a function of the expert count alone
+struct GateSplit {
+  int n_eb;    // expert blocks of 32 * kGateExpertBlocks
+  int parts;   // ranges of the contraction
+  int n_buf;   // partial tiles held in LDS at once
+};
+
+template <int V, int MT>
+__host__ __device__ inline GateSplit gate_split(int E) {
+  GateSplit sp;
+  sp.n_eb = (E + 32 * kGateExpertBlocks - 1) / (32 * kGateExpertBlocks);
+  sp.parts = kRouterWaves / sp.n_eb;
+  const int tile_bytes = MT * 32 * E * 4;
+  int fit = (kGateLdsBudget - GateShape<V>::kPartialBytes) / tile_bytes;
+  sp.n_buf = fit < 1 ? 1 : (fit > sp.parts ? sp.parts : fit);
+  return sp;
+}
 
 typedef float gate_f32x16_t __attribute__((ext_vector_type(16)));
 typedef __bf16 gate_bf16x8_t __attribute__((ext_vector_type(8)));
@@ -421,61 +461,125 @@ __device__ __forceinline__ gate_f32x16_t gate_mfma(f16_t, uint4 a, uint4 b, gate
                                                 0, 0);
 }
 
-// stage[tt * E + e] = logits of token t0 + tt (tt < 32) for every expert e; all threads take part.
-template <typename T>
+// stage[tt * E + e] = logits of token t0 + tt (tt < 32 * MT) for every expert e; all threads take part.
+template <typename T, int V, int MT>
 __device__ __forceinline__ void gate_tile(const GateArgs& g, int64_t t0, int64_t n_tokens, int E, float* stage) {
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int n_eb = (E + 31) / 32;         // 32-expert blocks (<= 16)
-  const int parts = kRouterWaves / n_eb;  // ranges of the contraction
-  const int eb = wave % n_eb, part = wave / n_eb;
-  if (part < parts) {
-    const int steps = g.hidden / 16;
-    const int per = (steps + parts - 1) / parts;
-    const int s0 = part * per, s1 = s0 + per < steps ? s0 + per : steps;
-    const int row = lane % 32, kc = (lane / 32) * 8;
-    const int64_t tok = t0 + row;
-    const int e = eb * 32 + row;
-    const bool live_a = tok < n_tokens, live_b = e < E;
-    const T* xa = static_cast<const T*>(g.x) + (live_a ? tok : 0) * g.hidden + kc;
-    const T* wb = static_cast<const T*>(g.w) + int64_t(live_b ? e : 0) * g.hidden + kc;
-    gate_f32x16_t acc;
+  constexpr int NT = kGateExpertBlocks, D = kGatePrefetch;
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // (uniform: step offsets stay scalar)
+  const GateSplit sp = gate_split<V, MT>(E);
+  const int eb = wave % sp.n_eb, part = wave / sp.n_eb;
+  const int tile_floats = MT * 32 * E;
+  const int row = lane % 32, half = lane / 32;
+  gate_f32x16_t acc[MT][NT];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-#pragma unroll 4
-    for (int st = s0; st < s1; ++st) {
-      const uint4 fa = live_a ? *reinterpret_cast<const uint4*>(xa + st * 16) : zero;
-      const uint4 fb = live_b ? *reinterpret_cast<const uint4*>(wb + st * 16) : zero;
-      acc = gate_mfma(T{}, fa, fb, acc);
-    }
-    // register 4*blk + q of lane l: token 8*blk + (l/32)*4 + q, expert eb*32 + l%32
-    float* tile = stage + part * (kGateTokens * E);
-    if (live_b) {
+  for (int m = 0; m < MT; ++m)
 #pragma unroll
-      for (int blk = 0; blk < 4; ++blk)
+    for (int n = 0; n < NT; ++n)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) tile[(8 * blk + (lane / 32) * 4 + q) * E + e] = acc[blk * 4 + q];
+      for (int r = 0; r < 16; ++r) acc[m][n][r] = 0.f;
+  if (part < sp.parts) {
+    // The contraction runs in batches of 64 elements, four matrix steps each.  A lane holds row
+    // lane % 32 and reads 64 contiguous bytes of that row's 128-byte line per batch (the lanes
+    // lane and lane + 32 share the line); x and the weights use the same positions along the
+    // contraction in every step, which is all a dot product asks for.
+    const int batches = g.hidden / 64;
+    const int per = (batches + sp.parts - 1) / sp.parts;
+    const int b0 = part * per;
+    const int steps = (b0 + per < batches ? per : batches - b0) * 4;
+    const uint32_t row_bytes = uint32_t(g.hidden) * uint32_t(sizeof(T));
+    const int64_t rows_left = n_tokens - t0;
+    const uint32_t live_rows = uint32_t(rows_left < MT * 32 ? rows_left : MT * 32);
+    // (buffer loads: a row past the end of x or of the weights reads as zero)
+    const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(static_cast<const T*>(g.x) + t0 * g.hidden), 0, int(live_rows * row_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(static_cast<const T*>(g.w)), 0, int(uint32_t(E) * row_bytes), 0x00020000);
+    uint32_t va[MT], vb[NT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) va[m] = uint32_t(m * 32 + row) * row_bytes + uint32_t(b0 * 128 + half * 64);
+#pragma unroll
+    for (int n = 0; n < NT; ++n) vb[n] = uint32_t((eb * NT + n) * 32 + row) * row_bytes + uint32_t(b0 * 128 + half * 64);
+    auto offset_of = [](int step) { return uint32_t((step >> 2) * 128 + (step & 3) * 16); };
+    auto fetch = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff) {
+      return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0));
+    };
+    uint4 fa[D][MT], fb[D][NT];
+    if (steps > 0) {
+      // (earlier stores drained here: with loads alone in flight the waits inside the loop can
+      // count them instead of draining everything)
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        const uint32_t off = offset_of(d < steps ? d : steps - 1);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) fa[d][m] = fetch(rsrc_x, va[m], off);
+#pragma unroll
+        for (int n = 0; n < NT; ++n) fb[d][n] = fetch(rsrc_w, vb[n], off);
+      }
+      for (int s0 = 0; s0 < steps; s0 += D) {  // steps is a multiple of 4, D divides 4
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n) acc[m][n] = gate_mfma(T{}, fa[d][m], fb[d][n], acc[m][n]);
+          const int nxt = s0 + d + D;  // (the last steps fetch the last step again: never used)
+          const uint32_t off = offset_of(nxt < steps ? nxt : steps - 1);
+#pragma unroll
+          for (int m = 0; m < MT; ++m) fa[d][m] = fetch(rsrc_x, va[m], off);
+#pragma unroll
+          for (int n = 0; n < NT; ++n) fb[d][n] = fetch(rsrc_w, vb[n], off);
+        }
+      }
     }
   }
-  __syncthreads();
-  for (int i = threadIdx.x; i < kGateTokens * E; i += kRouterWaves * kWave) {
+  // Partial tiles: part p adds into buffer p % n_buf in round p / n_buf, then the buffers are
+  // summed in order.  Register 4*blk + q of lane l: token 8*blk + (l/32)*4 + q, expert l%32.
+  const int rounds = (sp.parts + sp.n_buf - 1) / sp.n_buf;
+  const int my_round = part < sp.parts ? part / sp.n_buf : -1;
+  for (int r = 0; r < rounds; ++r) {
+    if (r == my_round) {
+      // (the index is made opaque so that the 16 * MT * NT addresses are formed here, one at a
+      // time, instead of being kept in registers across the chunk loop)
+      int first = (part % sp.n_buf) * tile_floats + half * 4 * E + eb * NT * 32 + row;
+      asm volatile("" : "+v"(first));
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        if ((eb * NT + n) * 32 + row < E) {
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                float* at = stage + first + n * 32 + (m * 32 + 8 * blk + q) * E;
+                *at = r == 0 ? acc[m][n][blk * 4 + q] : *at + acc[m][n][blk * 4 + q];
+              }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  for (int i = threadIdx.x; i < tile_floats; i += kRouterWaves * kWave) {
     float v = stage[i];
-    for (int q = 1; q < parts; ++q) v += stage[q * (kGateTokens * E) + i];
+    for (int q = 1; q < sp.n_buf; ++q) v += stage[q * tile_floats + i];
     stage[i] = g.fp32_logits ? v : to_float(from_float<T>(v));
   }
   __syncthreads();
 }
 
-template <int V, typename T>
+template <int V, typename T, int MT>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_gate_fwd_kernel(RouterArgs a, GateArgs g,
                                                                               int64_t* __restrict__ ids,
                                                                               float* __restrict__ weights,
                                                                               float* __restrict__ col_partial,
                                                                               int32_t* __restrict__ cnt_partial) {
   extern __shared__ __align__(16) unsigned char gate_smem[];
-  float* stage = reinterpret_cast<float*>(gate_smem);
-  float* lds_col = stage + kGateStageFloats;
+  constexpr int kTokens = MT * 32;
+  float* lds_col = reinterpret_cast<float*>(gate_smem);
   int32_t* lds_cnt = reinterpret_cast<int32_t*>(lds_col + kRouterWaves * V * kWave);
+  float* stage = reinterpret_cast<float*>(gate_smem + GateShape<V>::kPartialBytes);
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   float col[V];
@@ -488,16 +592,16 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_gate_fwd_kernel(Ro
   RouterArgs staged = a;  // the router reads this chunk's logits from LDS, as fp32
   staged.logits = stage;
   staged.logits_dtype = STM_F32;
-  for (int64_t t0 = int64_t(blockIdx.x) * kGateTokens; t0 < a.n_tokens; t0 += int64_t(gridDim.x) * kGateTokens) {
-    gate_tile<T>(g, t0, a.n_tokens, a.n_experts, stage);
-    for (int tt = wave; tt < kGateTokens; tt += kRouterWaves)
+  for (int64_t t0 = int64_t(blockIdx.x) * kTokens; t0 < a.n_tokens; t0 += int64_t(gridDim.x) * kTokens) {
+    gate_tile<T, V, MT>(g, t0, a.n_tokens, a.n_experts, stage);
+    for (int tt = wave; tt < kTokens; tt += kRouterWaves)
       if (t0 + tt < a.n_tokens) route_one<V>(staged, tt, t0 + tt, lane, ids, weights, col, cnt);
     __syncthreads();  // the next chunk overwrites the stage
   }
   write_partials<V>(col, cnt, lds_col, lds_cnt, a.n_experts, col_partial, cnt_partial);
 }
 
-template <int V, typename T>
+template <int V, typename T, int MT>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_gate_bwd_kernel(RouterArgs a, GateArgs g,
                                                                               const int64_t* __restrict__ ids,
                                                                               const float* __restrict__ grad_w,
@@ -506,6 +610,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_gate_bwd_kernel(Ro
                                                                               void* __restrict__ grad_logits,
                                                                               int grad_dtype) {
   extern __shared__ __align__(16) unsigned char gate_smem[];
+  constexpr int kTokens = MT * 32;
   float* stage = reinterpret_cast<float*>(gate_smem);
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
@@ -514,23 +619,31 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_gate_bwd_kernel(Ro
   RouterArgs staged = a;
   staged.logits = stage;
   staged.logits_dtype = STM_F32;
-  for (int64_t t0 = int64_t(blockIdx.x) * kGateTokens; t0 < a.n_tokens; t0 += int64_t(gridDim.x) * kGateTokens) {
-    gate_tile<T>(g, t0, a.n_tokens, a.n_experts, stage);
-    for (int tt = wave; tt < kGateTokens; tt += kRouterWaves)
+  for (int64_t t0 = int64_t(blockIdx.x) * kTokens; t0 < a.n_tokens; t0 += int64_t(gridDim.x) * kTokens) {
+    gate_tile<T, V, MT>(g, t0, a.n_tokens, a.n_experts, stage);
+    for (int tt = wave; tt < kTokens; tt += kRouterWaves)
       if (t0 + tt < a.n_tokens) route_one_bwd<V>(staged, tt, t0 + tt, lane, ids, grad_w, dcol, grad_logits, grad_dtype);
     __syncthreads();
   }
 }
 
-inline int gate_blocks(int64_t n_tokens) {
-  const int64_t want = (n_tokens + kGateTokens - 1) / kGateTokens;
+// workgroups of a launch: one per chunk, at most 512 (never more than router_blocks(), which sizes
+// the workspace of partial rows)
+inline int gate_blocks(int64_t n_tokens, int n_experts) {
+  const int chunk = 32 * gate_token_blocks(n_experts);
+  const int64_t want = (n_tokens + chunk - 1) / chunk;
   return int(want < 1 ? 1 : (want > 512 ? 512 : want));
 }
 
-// shapes the fused gate takes: 16-bit elements, hidden a multiple of 16, at most 512 experts
+template <int V, int MT>
+inline size_t gate_stage_bytes(int E) {
+  return size_t(gate_split<V, MT>(E).n_buf) * MT * 32 * E * 4;
+}
+
+// shapes the fused gate takes: 16-bit elements, hidden a multiple of 64, at most 512 experts
 inline int check_gate_args(const void* x, const void* w, int dtype, int hidden, int n_experts) {
   if (dtype != STM_BF16 && dtype != STM_F16) return STM_ERR_UNSUPPORTED;
-  if (hidden <= 0 || hidden % 16 != 0 || n_experts > 32 * kRouterWaves) return STM_ERR_UNSUPPORTED;
+  if (hidden <= 0 || hidden % 64 != 0 || n_experts > 32 * kRouterWaves) return STM_ERR_UNSUPPORTED;
   if (!aligned_to(x, 16) || !aligned_to(w, 16)) return STM_ERR_UNSUPPORTED;
   return STM_OK;
 }
@@ -543,23 +656,44 @@ int allow_large_lds(K kernel, size_t bytes) {
              : STM_ERR_LAUNCH;
 }
 
+template <int V, typename T, int MT>
+int launch_gate_fwd_as(const RouterArgs& a, const GateArgs& g, int blocks, int64_t* ids, float* weights,
+                       float* col_partial, int32_t* cnt_partial, hipStream_t s) {
+  const size_t lds = gate_stage_bytes<V, MT>(a.n_experts) + GateShape<V>::kPartialBytes;
+  if (allow_large_lds(router_gate_fwd_kernel<V, T, MT>, lds) != STM_OK) return STM_ERR_LAUNCH;
+  router_gate_fwd_kernel<V, T, MT><<<blocks, kRouterWaves * kWave, lds, s>>>(a, g, ids, weights, col_partial, cnt_partial);
+  return STM_OK;
+}
+
+template <int V, typename T, int MT>
+int launch_gate_bwd_as(const RouterArgs& a, const GateArgs& g, int blocks, const int64_t* ids, const float* grad_w,
+                       const float* grad_aux, const int32_t* hist, void* grad_logits, int grad_dtype, hipStream_t s) {
+  const size_t lds = gate_stage_bytes<V, MT>(a.n_experts);
+  if (allow_large_lds(router_gate_bwd_kernel<V, T, MT>, lds) != STM_OK) return STM_ERR_LAUNCH;
+  router_gate_bwd_kernel<V, T, MT><<<blocks, kRouterWaves * kWave, lds, s>>>(a, g, ids, grad_w, grad_aux, hist, grad_logits,
+                                                                             grad_dtype);
+  return STM_OK;
+}
+
+// (only rows of 257 to 512 experts come in both chunk sizes)
 template <int V, typename T>
 int launch_gate_fwd(const RouterArgs& a, const GateArgs& g, int blocks, int64_t* ids, float* weights, float* col_partial,
                     int32_t* cnt_partial, hipStream_t s) {
-  const size_t lds = size_t(kGateStageFloats) * 4 + size_t(kRouterWaves) * V * kWave * 8;
-  if (allow_large_lds(router_gate_fwd_kernel<V, T>, lds) != STM_OK) return STM_ERR_LAUNCH;
-  router_gate_fwd_kernel<V, T><<<blocks, kRouterWaves * kWave, lds, s>>>(a, g, ids, weights, col_partial, cnt_partial);
-  return STM_OK;
+  if constexpr (V <= 4) return launch_gate_fwd_as<V, T, 2>(a, g, blocks, ids, weights, col_partial, cnt_partial, s);
+  if constexpr (V == 8)
+    if (gate_token_blocks(a.n_experts) == 2)
+      return launch_gate_fwd_as<V, T, 2>(a, g, blocks, ids, weights, col_partial, cnt_partial, s);
+  return launch_gate_fwd_as<V, T, 1>(a, g, blocks, ids, weights, col_partial, cnt_partial, s);
 }
 
 template <int V, typename T>
 int launch_gate_bwd(const RouterArgs& a, const GateArgs& g, int blocks, const int64_t* ids, const float* grad_w,
                     const float* grad_aux, const int32_t* hist, void* grad_logits, int grad_dtype, hipStream_t s) {
-  const size_t lds = size_t(kGateStageFloats) * 4;
-  if (allow_large_lds(router_gate_bwd_kernel<V, T>, lds) != STM_OK) return STM_ERR_LAUNCH;
-  router_gate_bwd_kernel<V, T><<<blocks, kRouterWaves * kWave, lds, s>>>(a, g, ids, grad_w, grad_aux, hist, grad_logits,
-                                                                         grad_dtype);
-  return STM_OK;
+  if constexpr (V <= 4) return launch_gate_bwd_as<V, T, 2>(a, g, blocks, ids, grad_w, grad_aux, hist, grad_logits, grad_dtype, s);
+  if constexpr (V == 8)
+    if (gate_token_blocks(a.n_experts) == 2)
+      return launch_gate_bwd_as<V, T, 2>(a, g, blocks, ids, grad_w, grad_aux, hist, grad_logits, grad_dtype, s);
+  return launch_gate_bwd_as<V, T, 1>(a, g, blocks, ids, grad_w, grad_aux, hist, grad_logits, grad_dtype, s);
 }
 
 // Aux-loss-free load balancing: bias[e] += sign(mean(tokens) - tokens[e]) * rate, then the token
@@ -681,11 +815,11 @@ int stm_router_gate_fwd(const void* x, const void* gate_w, int dtype, int hidden
   if (n_tokens > 0 && top_k > 0 && (!ids_out || !weights_out)) return STM_ERR_ARG;
   if (workspace_bytes < stm_router_workspace_bytes(n_tokens, n_experts) || !workspace) return STM_ERR_WORKSPACE;
   hipStream_t s = as_stream(stream);
-  const int blocks = gate_blocks(n_tokens);  // never more than router_blocks(): the workspace holds the partial rows
+  const int need = (n_experts + kWave - 1) / kWave;
+  const int blocks = gate_blocks(n_tokens, n_experts);
   float* col_partial = static_cast<float*>(workspace);
   int32_t* cnt_partial = reinterpret_cast<int32_t*>(col_partial + size_t(blocks) * n_experts);
   GateArgs g{x, gate_w, hidden, fp32_logits};
-  const int need = (n_experts + kWave - 1) / kWave;
   if (dtype == STM_BF16) {
     STM_ROUTER_DISPATCH(need, (st = launch_gate_fwd<V, bf16_t>(a, g, blocks, ids_out, weights_out, col_partial, cnt_partial, s)));
   } else {
@@ -711,9 +845,9 @@ int stm_router_gate_bwd(const void* x, const void* gate_w, int dtype, int hidden
   st = check_gate_args(x, gate_w, dtype, hidden, n_experts);
   if (st != STM_OK) return st;
   hipStream_t s = as_stream(stream);
-  const int blocks = gate_blocks(n_tokens);
   GateArgs g{x, gate_w, hidden, fp32_logits};
   const int need = (n_experts + kWave - 1) / kWave;
+  const int blocks = gate_blocks(n_tokens, n_experts);
   if (dtype == STM_BF16) {
     STM_ROUTER_DISPATCH(need, (st = launch_gate_bwd<V, bf16_t>(a, g, blocks, ids, grad_weights, grad_aux_or_null, hist, grad_logits, grad_dtype, s)));
   } else {

@@ -151,7 +151,7 @@ def gate_router_takes(x: torch.Tensor, gate_w: torch.Tensor) -> bool:
     """Shapes the fused gate + router kernel takes (others compute the logits first)."""
     return (
         x.is_cuda and x.dim() == 2 and x.dtype in (torch.bfloat16, torch.float16) and gate_w.dtype == x.dtype
-        and x.shape[1] % 16 == 0 and gate_w.shape[0] <= 512 and gate_w.shape[1] == x.shape[1]
+        and x.shape[1] % 64 == 0 and gate_w.shape[0] <= 512 and gate_w.shape[1] == x.shape[1]
     )  # fmt: skip
 
 
@@ -298,7 +298,10 @@ class MoEBlock(nn.Module):
         the sum of both, the scaling and the addition done by the combine kernel."""
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
-        if logits is None and settings.fuse_gate and gate_router_takes(x2, self.gate.weight):
+        # (a 16-bit gate output is faster as library GEMM + router; the fused kernel wins where the
+        # reference's gate would copy x and the weights to fp32 first)
+        fuse = settings.fuse_gate == "always" or (settings.fuse_gate and self.gate.fp32_output)
+        if logits is None and fuse and gate_router_takes(x2, self.gate.weight):
             ids, weights, aux, hist = forward_gate_router(
                 x2, self.gate.weight, self.top_k, fp32_output=self.gate.fp32_output, use_sigmoid=self.use_sigmoid_router,
                 norm_expert_weight=self.norm_expert_weight, balance_bias=self.router_balance_bias, n_group=self.n_group,

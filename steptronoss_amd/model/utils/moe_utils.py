@@ -65,9 +65,10 @@ class Settings:
         (the fp8 benchmark configuration; no counterpart in the reference): activations are quantised
         on the way into each GEMM, the weights once per weight version, in both orientations.
         Weight gradients stay in the tensors' own dtype.
-    fuse_gate: ``MoEBlock`` computes the gate GEMM inside the router kernel (bf16 / fp16, hidden a
-        multiple of 16, at most 512 experts), so the logits never reach HBM; off: ``MoEGate`` then the
-        router, as two steps.
+    fuse_gate: ``MoEBlock`` with an fp32 gate output computes the gate GEMM inside the router kernel
+        (bf16 / fp16 inputs, hidden a multiple of 64, at most 512 experts): the logits never reach
+        HBM and no fp32 copies of the inputs are made.  ``"always"``: 16-bit gate outputs as well
+        (there library GEMM + router is the faster pair).  Off: ``MoEGate`` then the router.
     deferred_id_check: ``routed_grouped_ffn`` copies the routing status words to pinned host
         memory without waiting; a later call (or ``check_deferred_status()``) that finds such a
         copy complete raises the reference's "out-of-range" ``ValueError`` for an expert id
@@ -81,7 +82,7 @@ class Settings:
     probe_activation: bool = False
     deferred_id_check: bool = True
     fp8_experts: bool = False
-    fuse_gate: bool = True
+    fuse_gate: bool | str = True
 
 
 settings = Settings()
