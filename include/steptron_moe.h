@@ -265,13 +265,36 @@ int stm_grouped_gemm_dswiglu(const void* grad_y, const void* w2, const void* gat
                              int64_t m_cap, int ffn, int k, int has_limit, float limit, int dtype, void* workspace,
                              size_t workspace_bytes, stm_stream_t stream);
 
+/* The fused products with their row operand GATHERED instead of copied first: row r of the
+ * operand is row row_sources[r] of src [src_rows_n, k] (row_sources int32, from
+ * stm_slot_tokens_to_rows: m_cap entries followed by stm_row_sources_padding() readable
+ * entries of any content, which let the kernels fetch the table in blocks).  They replace moe_scatter's copy of x (moe_utils.py:339-374, called at
+ * :226) in front of the first expert GEMM, and the copy of grad_out in front of the second
+ * GEMM's input gradient: the GEMM's loads read the token rows themselves.  Results are those of
+ * stm_permute_fwd followed by the entry without "_gathered", bit for bit.  STM_ERR_UNSUPPORTED
+ * additionally when src is 2 GiB or larger, or (swiglu) k is not a multiple of 64. */
+int stm_row_sources_padding(void);
+int stm_grouped_gemm_swiglu_gathered(const void* src, int64_t src_rows_n, const int32_t* row_sources, const void* w1,
+                                     void* gate_up, void* h, const float* row_scale, const int32_t* offsets,
+                                     int n_groups, int64_t m_cap, int ffn, int k, int has_limit, float limit, int dtype,
+                                     void* workspace, size_t workspace_bytes, stm_stream_t stream);
+int stm_grouped_gemm_dswiglu_gathered(const void* src, int64_t src_rows_n, const int32_t* row_sources, const void* w2,
+                                      const void* gate_up, void* grad_gate_up, const float* row_scale, float* row_dot,
+                                      const int32_t* offsets, int n_groups, int64_t m_cap, int ffn, int k,
+                                      int has_limit, float limit, int dtype, void* workspace, size_t workspace_bytes,
+                                      stm_stream_t stream);
+
 /* Between slot order ([T, K], token-major) and row order (pos = index_compute's output):
+ *   stm_slot_tokens_to_rows: token_of_row[pos[s]] = s / top_k for every slot with pos[s] >= 0
+ *                            (int32 [n_rows]; the row_sources of the gathered products);
  *   stm_slot_values_to_rows: rows[pos[s]] = float(values[s]) for every slot with pos[s] >= 0
  *                            (values: fp32/fp16/bf16 by value_dtype; rows fp32 [n_rows]);
  *   stm_row_parts_to_slots : out[s] = sum_p parts[pos[s], p] (0 for pos[s] < 0), parts fp32
  *                            [n_rows, n_parts], out in out_dtype.
  * Together with row_scale / row_dot above they carry token_weights into the fused expert FFN
  * and its gradient back (no counterpart in the reference, which weights in the combine). */
+int stm_slot_tokens_to_rows(const int32_t* pos, int64_t n_slots, int top_k, int32_t* token_of_row, int64_t n_rows,
+                            stm_stream_t stream);
 int stm_slot_values_to_rows(const void* values, int value_dtype, const int32_t* pos, int64_t n_slots, float* rows,
                             int64_t n_rows, stm_stream_t stream);
 int stm_row_parts_to_slots(const float* parts, int n_parts, const int32_t* pos, int64_t n_slots, int64_t n_rows,
@@ -281,6 +304,17 @@ int stm_row_parts_to_slots(const float* parts, int n_parts, const int32_t* pos, 
  * x:[m_cap, p], y:[m_cap, q], out:[G, p, q]; an empty group gives zeros (:56-58). */
 int stm_grouped_gemm_wgrad(const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
                            int64_t m_cap, int p, int q, int dtype, stm_stream_t stream);
+
+/* The same product with one operand gathered: gathered_operand 1: x, 2: y; row r of that
+ * operand is row row_sources[r] of the buffer passed for it, which has src_rows_n rows
+ * (the other operand has m_cap rows, row_sources m_cap entries plus the padding named above).
+ * Serves the weight gradients of the
+ * expert FFN without the permuted copies of x and grad_out (moe_utils.py:226,
+ * function_imple.py:54-69).  bf16 / fp16, p and q at least 256 and multiples of 8, the gathered
+ * buffer below 2 GiB; STM_ERR_UNSUPPORTED otherwise (the caller then copies the rows first). */
+int stm_grouped_gemm_wgrad_gathered(const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
+                                    int64_t m_cap, int p, int q, int dtype, const int32_t* row_sources,
+                                    int gathered_operand, int64_t src_rows_n, stm_stream_t stream);
 
 /* The same product ADDED to an fp32 buffer accum [G, p, q] instead of stored in the operands'
  * dtype: the weight gradient accumulated straight into the optimizer's fp32 "main_grad"

@@ -67,6 +67,11 @@ SIGNATURES = {
     "stm_grouped_gemm_swiglu": (I, [P, P, P, P, P, P, I, L, I, I, I, F, I, P, Z, P]),
     "stm_grouped_gemm_dswiglu_row_dot_parts": (I, [I]),
     "stm_grouped_gemm_dswiglu": (I, [P, P, P, P, P, P, P, I, L, I, I, I, F, I, P, Z, P]),
+    "stm_grouped_gemm_swiglu_gathered": (I, [P, L, P, P, P, P, P, P, I, L, I, I, I, F, I, P, Z, P]),
+    "stm_grouped_gemm_dswiglu_gathered": (I, [P, L, P, P, P, P, P, P, P, I, L, I, I, I, F, I, P, Z, P]),
+    "stm_grouped_gemm_wgrad_gathered": (I, [P, P, P, P, I, L, I, I, I, P, I, L, P]),
+    "stm_slot_tokens_to_rows": (I, [P, L, I, P, L, P]),
+    "stm_row_sources_padding": (I, []),
     "stm_slot_values_to_rows": (I, [P, I, P, L, P, L, P]),
     "stm_row_parts_to_slots": (I, [P, I, P, L, L, P, I, P]),
     "stm_quantize_e4m3_1x128": (I, [P, I, L, L, P, P, P]),

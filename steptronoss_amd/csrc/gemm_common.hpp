@@ -91,6 +91,14 @@ struct GemmArgs {
   const float* a_scales;
   const float* b_scales;
   int64_t a_scale_rows, b_scale_rows;
+  // Gathered operand (null: none): row r of that operand is row src_rows[r] of the buffer given
+  // for it (r counts as the offsets do), so that the rows of a permuted copy are read straight
+  // from the tensor they would have been copied from.  gather_operand: 1 = a, 2 = b (wgrad form
+  // only); src_bytes: size of that buffer (below 2^31); src_n_rows: entries of src_rows.
+  const int32_t* src_rows;
+  int64_t src_n_rows;
+  uint32_t src_bytes;
+  int gather_operand;
 };
 
 // Fused SwiGLU forms of the rows GEMM (gemm_mfma_dma.hip); STM_ERR_UNSUPPORTED when the shape does not fit.

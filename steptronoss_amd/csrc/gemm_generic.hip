@@ -13,7 +13,8 @@ namespace stm {
 int launch_mfma_rows(int dtype, const void* a, const void* b, void* c, const int32_t* offsets, int n_groups,
                      int64_t m_cap, int n, int k, int b_is_nk, void* ws, size_t ws_bytes, hipStream_t s);
 int launch_mfma_wgrad(int dtype, const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
-                      int64_t m_cap, int p, int q, int accumulate, hipStream_t s);
+                      int64_t m_cap, int p_dim, int q_dim, int accumulate, hipStream_t s,
+                      const int32_t* src_rows = nullptr, int gather_operand = 0, int64_t src_buffer_rows = 0);
 
 namespace {
 
@@ -305,6 +306,81 @@ int stm_grouped_gemm_wgrad(const void* x, const void* y, void* out, const int32_
   p.wgrad = 1;
   dim3 grid(unsigned((q_dim + kGT - 1) / kGT), unsigned((p_dim + kGT - 1) / kGT), unsigned(n_groups));
   return dispatch_generic(dtype, p, grid, s);
+}
+
+namespace {
+// The gathered operand of a fused entry: rows of `src` [src_rows_n, k] named by row_sources [m_cap].
+int gathered_source(stm::GemmArgs& p, const int32_t* row_sources, int64_t src_rows_n, int k, int64_t m_cap) {
+  if (!row_sources || src_rows_n < 0) return STM_ERR_ARG;
+  const int64_t bytes = src_rows_n * int64_t(k) * 2;
+  if (bytes <= 0 || bytes >= (int64_t(1) << 31)) return STM_ERR_UNSUPPORTED;
+  p.src_rows = row_sources;
+  p.src_n_rows = m_cap;
+  p.src_bytes = uint32_t(bytes);
+  p.gather_operand = 1;
+  return STM_OK;
+}
+}  // namespace
+
+int stm_row_sources_padding(void) { return 512; }
+
+int stm_grouped_gemm_swiglu_gathered(const void* src, int64_t src_rows_n, const int32_t* row_sources, const void* w1,
+                                     void* gate_up, void* h, const float* row_scale, const int32_t* offsets,
+                                     int n_groups, int64_t m_cap, int ffn, int k, int has_limit, float limit, int dtype,
+                                     void* workspace, size_t workspace_bytes, stm_stream_t stream) {
+  using namespace stm;
+  GemmArgs p;
+  int st = fused_args(src, w1, gate_up, h, offsets, n_groups, m_cap, ffn, k, has_limit, limit, dtype, workspace,
+                      workspace_bytes, p);
+  if (st != STM_OK) return st;
+  st = gathered_source(p, row_sources, src_rows_n, k, m_cap);
+  if (st != STM_OK) return st;
+  p.lda = k;
+  p.ldb = k;
+  p.ldc = 2 * int64_t(ffn);
+  p.ldc2 = ffn;
+  p.b_group = 2 * int64_t(ffn) * k;
+  p.n_j = 2 * ffn;
+  p.n_k = k;
+  p.row_scale = row_scale;
+  return launch_dma_swiglu_fwd(dtype, p, offsets, n_groups, m_cap, workspace, as_stream(stream));
+}
+
+int stm_grouped_gemm_dswiglu_gathered(const void* src, int64_t src_rows_n, const int32_t* row_sources, const void* w2,
+                                      const void* gate_up, void* grad_gate_up, const float* row_scale, float* row_dot,
+                                      const int32_t* offsets, int n_groups, int64_t m_cap, int ffn, int k,
+                                      int has_limit, float limit, int dtype, void* workspace, size_t workspace_bytes,
+                                      stm_stream_t stream) {
+  using namespace stm;
+  GemmArgs p;
+  int st = fused_args(src, w2, grad_gate_up, const_cast<void*>(gate_up), offsets, n_groups, m_cap, ffn, k, has_limit,
+                      limit, dtype, workspace, workspace_bytes, p);
+  if (st != STM_OK) return st;
+  st = gathered_source(p, row_sources, src_rows_n, k, m_cap);
+  if (st != STM_OK) return st;
+  p.lda = k;
+  p.ldb = ffn;
+  p.ldc = 2 * int64_t(ffn);
+  p.ldc2 = 2 * int64_t(ffn);
+  p.b_group = int64_t(ffn) * k;
+  p.n_j = ffn;
+  p.n_k = k;
+  p.row_scale = row_scale;
+  p.row_dot = row_dot;
+  return launch_dma_swiglu_bwd(dtype, p, offsets, n_groups, m_cap, workspace, as_stream(stream));
+}
+
+int stm_grouped_gemm_wgrad_gathered(const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
+                                    int64_t m_cap, int p_dim, int q_dim, int dtype, const int32_t* row_sources,
+                                    int gathered_operand, int64_t src_rows_n, stm_stream_t stream) {
+  using namespace stm;
+  if (n_groups < 0 || m_cap < 0 || p_dim < 0 || q_dim < 0 || src_rows_n < 0) return STM_ERR_ARG;
+  if (gathered_operand != 1 && gathered_operand != 2) return STM_ERR_ARG;
+  if ((dtype != STM_BF16 && dtype != STM_F16) || n_groups > kMaxGroups) return STM_ERR_UNSUPPORTED;
+  if (n_groups == 0 || p_dim == 0 || q_dim == 0 || m_cap == 0) return STM_ERR_UNSUPPORTED;
+  if (!out || !offsets || !x || !y || !row_sources) return STM_ERR_ARG;
+  return launch_mfma_wgrad(dtype, x, y, out, offsets, n_groups, m_cap, p_dim, q_dim, 0, as_stream(stream), row_sources,
+                           gathered_operand, src_rows_n);
 }
 
 }  // extern "C"

@@ -337,7 +337,8 @@ int launch_mfma_rows(int dtype, const void* a, const void* b, void* c, const int
 
 // accumulate != 0: `out` is an fp32 buffer the product is added to (only the 256 x 256 kernels do that).
 int launch_mfma_wgrad(int dtype, const void* x, const void* y, void* out, const int32_t* offsets, int n_groups,
-                      int64_t m_cap, int p_dim, int q_dim, int accumulate, hipStream_t s) {
+                      int64_t m_cap, int p_dim, int q_dim, int accumulate, hipStream_t s, const int32_t* src_rows,
+                      int gather_operand, int64_t src_buffer_rows) {
   (void)m_cap;
   if (dtype != STM_BF16 && dtype != STM_F16) return STM_ERR_UNSUPPORTED;
   if (p_dim % 8 != 0 || q_dim % 8 != 0) return STM_ERR_UNSUPPORTED;
@@ -354,6 +355,15 @@ int launch_mfma_wgrad(int dtype, const void* x, const void* y, void* out, const 
   p.n_i = p_dim;
   p.n_j = q_dim;
   p.n_groups = n_groups;
+  if (src_rows) {  // a gathered operand: the persistent kernel or nothing
+    const int64_t bytes = src_buffer_rows * (gather_operand == 2 ? q_dim : p_dim) * 2;
+    if (p_dim < 256 || q_dim < 256 || bytes <= 0 || bytes >= (int64_t(1) << 31)) return STM_ERR_UNSUPPORTED;
+    p.src_rows = src_rows;
+    p.src_n_rows = m_cap;
+    p.src_bytes = uint32_t(bytes);
+    p.gather_operand = gather_operand;
+    return launch_dma_wgrad(dtype, p, n_groups, m_cap, accumulate, s);
+  }
   if (p_dim >= 256 && q_dim >= 256) {
     const int st = launch_dma_wgrad(dtype, p, n_groups, m_cap, accumulate, s);
     if (st != STM_ERR_UNSUPPORTED) return st;

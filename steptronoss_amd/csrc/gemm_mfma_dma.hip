@@ -136,6 +136,8 @@ struct OperandPlan {
   static_assert(kLoadsPerWave % 2 == 0, "the parity trick needs an even number of loads per wave");
   static_assert(!KM || kRowsPerLoad == 2 || kRowsPerLoad == 4, "KM tiles of 128 or 256 columns");
   uint32_t voff[2];      // lane offset for even / odd loads, relative to the load's first row
+  uint32_t col[2];       // the same without the row part (a gathered operand adds its own row offset)
+  int row_in_load;       // stored row of this lane inside a load
   uint32_t load_stride;  // bytes between the first rows of consecutive loads
   uint32_t step_bytes;   // scalar offset increment per contraction step
 
@@ -147,21 +149,26 @@ struct OperandPlan {
         if constexpr (kBK == 64) {
           // stored row r = load*8 + lane/8 (128 bytes), chunk = (lane%8) ^ ((r >> 1) & 7)
           const int sw = ((parity * 4) + lane / 16) & 7;
-          voff[parity] = uint32_t(lane / 8) * row_bytes + uint32_t((lane % 8) ^ sw) * 16u;
+          row_in_load = lane / 8;
+          col[parity] = uint32_t((lane % 8) ^ sw) * 16u;
+          voff[parity] = uint32_t(row_in_load) * row_bytes + col[parity];
         } else {
           // stored row r = load*16 + lane/4 (64 bytes), chunk = (lane%4) ^ ((r >> 2) & 3): the
           // swizzle does not depend on the load
           const int sw = (lane / 16) & 3;
-          voff[parity] = uint32_t(lane / 4) * row_bytes + uint32_t((lane % 4) ^ sw) * 16u;
+          row_in_load = lane / 4;
+          col[parity] = uint32_t((lane % 4) ^ sw) * 16u;
+          voff[parity] = uint32_t(row_in_load) * row_bytes + col[parity];
         }
       } else {
         // stored row k = load*kRowsPerLoad + lane/(R/8), 64-byte chunk = (c16/4) ^ (k & 3)
         constexpr int kChunks16 = R / 8;
-        const int row_in_load = lane / kChunks16;
+        row_in_load = lane / kChunks16;
         const int c16 = lane % kChunks16;
         const int k_low = ((parity * kRowsPerLoad) + row_in_load) & 3;
-        const int col = (((c16 / 4) ^ k_low) * 32) + (c16 % 4) * 8;
-        voff[parity] = uint32_t(row_in_load) * row_bytes + uint32_t(col) * 2u;
+        const int col_elems = (((c16 / 4) ^ k_low) * 32) + (c16 % 4) * 8;
+        col[parity] = uint32_t(col_elems) * 2u;
+        voff[parity] = uint32_t(row_in_load) * row_bytes + col[parity];
       }
     }
     load_stride = __builtin_amdgcn_readfirstlane(uint32_t(kRowsPerLoad) * row_bytes);
@@ -182,6 +189,17 @@ struct OperandPlan {
     uint32_t soff = __builtin_amdgcn_readfirstlane(soff0 + uint32_t(j) * load_stride);
     asm volatile("" : "+s"(soff));  // keep it in an SGPR: a folded literal is not a legal soffset
     dma16(rsrc, __builtin_amdgcn_readfirstlane(lds_wave_addr + uint32_t(j) * 1024u), voff[j & 1], soff);
+  }
+  // the same for a gathered operand: the lane offset names the source row (and the column), the
+  // scalar offset is the same for all loads of the stage
+  __device__ __forceinline__ void issue_gathered(i32x4_t rsrc_in, uint32_t lds_wave_addr, uint32_t soff_in, int j,
+                                                 uint32_t voffset) const {
+    i32x4_t rsrc;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) rsrc[w] = __builtin_amdgcn_readfirstlane(rsrc_in[w]);
+    uint32_t soff = __builtin_amdgcn_readfirstlane(soff_in);
+    asm volatile("" : "+s"(soff));
+    dma16(rsrc, __builtin_amdgcn_readfirstlane(lds_wave_addr + uint32_t(j) * 1024u), voffset, soff);
   }
 };
 
@@ -217,6 +235,10 @@ struct TileState {
   int row0;          // rows form: first row of the tile in the whole problem
   int64_t brow0;     // rows form: row of the tile's first column in b seen as [G * n_j, k]
   int valid_i, valid_j, n_steps;
+  // gathered operand: first row and row count of the tile (rows form) or group (wgrad) in
+  // src_rows, scalar byte offset of the tile's first column
+  int g_lo, g_nk;
+  uint32_t g_soff;
 };
 
 // What the epilogue does with the accumulators.
@@ -250,7 +272,13 @@ enum Epilogue { kStore = 0, kSwigluFwd = 1, kSwigluBwd = 2, kAccumF32 = 3, kStor
 // after both, so that between two barriers one multiplies while the other reads and then they
 // swap: the matrix pipe is fed back to back, no MFMA waits for an LDS read of its own wave,
 // and the epilogue of one wave runs under the MFMAs of its partner.
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int kBK, int EPI, bool PP>
+// GATHER = 1 / 2: the rows of operand a / b (b: wgrad only) are read through p.src_rows.  The
+// loads keep their number, order and LDS destinations; only the lane offsets change, so nothing
+// of the pipeline's bookkeeping does.  The row numbers come in through scalar loads (rows form:
+// the 32 rows a wave loads, once per tile; wgrad: the 4 contraction rows a wave loads, once
+// per step, fetched a step ahead).
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int kBK, int EPI, bool PP,
+          int GATHER>
 __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs p) {
   static_assert(kBK == 64 || kBK == 32, "contraction elements per stage");
   static_assert(!PP || (WAVES == 8 && kBK == 32 && EPI != kStoreFp8), "ping-pong: 8 waves, stages of 32");
@@ -281,6 +309,16 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   // loads that may still be in flight at the barrier of step g: those of stages g+2 .. g+kStages-1
   constexpr int kInFlight = (kStages - 2) * kLoads;
   static_assert(kInFlight < 64, "vmcnt is a 6-bit counter");
+  constexpr bool kGatherA = GATHER == 1, kGatherB = GATHER == 2;
+  static_assert(GATHER == 0 || !kFp8, "no gathered fp8 operands");
+  static_assert(!kGatherB || WGRAD, "the rows form gathers its a operand");
+  static_assert(!(kGatherA && !WGRAD) || (!A_KM && PlanA::kLoadsPerWave * PlanA::kRowsPerLoad == 32),
+                "rows form: a wave loads 32 consecutive rows of the tile");
+  static_assert(!(GATHER != 0 && WGRAD) || (PlanA::kLoadsPerWave == 2 && PlanA::kRowsPerLoad == 2 &&
+                                            PlanB::kLoadsPerWave == 2 && PlanB::kRowsPerLoad == 2),
+                "wgrad: a wave loads 4 consecutive contraction rows per stage");
+  constexpr int kLoadsG = GATHER == 0 ? 1 : (kGatherB ? kLoadsB : kLoadsA);
+  constexpr uint32_t kGatherDropped = 0x80000000u;  // past the end of any gathered buffer: reads as zero
   static_assert(BN == 256 && sizeof(T) == 2 && (kStageCols == 128 || kStageCols == 64),
                 "epilogue staging assumes 128 columns of 16-bit outputs per wave, staged 128 or 64 at a time");
   extern __shared__ __align__(1024) unsigned char smem[];
@@ -378,8 +416,11 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       n_k = hi > lo ? int(hi - lo) : 0;
       const int i0 = it * BM;
       t.valid_i = p.n_i - i0;
-      a += lo * p.lda + i0;
-      b += lo * p.ldb + j0;
+      if constexpr (!kGatherA) a += lo * p.lda + i0;
+      if constexpr (!kGatherB) b += lo * p.ldb + j0;
+      t.g_lo = int(lo);
+      t.g_nk = n_k;
+      t.g_soff = uint32_t(kGatherB ? j0 : i0) * 2u;
       if constexpr (EPI == kAccumF32)
         c = reinterpret_cast<T*>(static_cast<float*>(p.c) + g * p.c_group + int64_t(i0) * p.ldc + j0);
       else
@@ -387,18 +428,21 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
       // contraction rows past the end of the group are past the end of the buffer: zeros
       const int64_t ab = int64_t(n_k) * p.lda * 2 - int64_t(i0) * 2;
       const int64_t bb = int64_t(n_k) * p.ldb * 2 - int64_t(j0) * 2;
-      a_bytes = ab > 0 ? uint32_t(ab) : 0u;
-      b_bytes = bb > 0 ? uint32_t(bb) : 0u;
+      a_bytes = kGatherA ? p.src_bytes : ab > 0 ? uint32_t(ab) : 0u;
+      b_bytes = kGatherB ? p.src_bytes : bb > 0 ? uint32_t(bb) : 0u;
     } else {
       const MTile mt = scalar_load(p.tiles, id_over_j);
       n_k = p.n_k;
       t.valid_i = mt.rows;
       t.row0 = mt.row0;
       t.brow0 = int64_t(mt.group) * p.n_j + j0;
-      a += int64_t(mt.row0) * p.lda;
+      if constexpr (!kGatherA) a += int64_t(mt.row0) * p.lda;
+      t.g_lo = mt.row0;
+      t.g_nk = mt.rows;
+      t.g_soff = 0;
       c += int64_t(mt.row0) * p.ldc + (EPI == kStore || EPI == kStoreFp8 ? j0 : 0);
       if constexpr (EPI != kStore && EPI != kStoreFp8) t.c2 = static_cast<T*>(p.c2) + int64_t(mt.row0) * p.ldc2;
-      a_bytes = uint32_t(int64_t(mt.rows) * p.lda * 2);
+      a_bytes = kGatherA ? p.src_bytes : uint32_t(int64_t(mt.rows) * p.lda * 2);
       if constexpr (EPI == kSwigluFwd) {
         // the descriptor covers all 2*ffn rows of the expert's W1; this wave's 32 tile rows are
         // one run of gate rows or of up rows
@@ -444,7 +488,73 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   // keeps going with an empty descriptor: such loads move no data (and write zeros to an LDS
   // slot nobody reads any more), which keeps the steady-state code free of branches.
   i32x4_t l_rsrc_a, l_rsrc_b;
-  const uint32_t l_soff_a0 = plan_a.stage_soffset(0, wave);
+  // gathered operand: lane offsets of the loads of the stage under the cursor, and the scalars
+  // they are made from
+  uint32_t g_voff[kLoadsG];
+  int g_bank = 0;  // wgrad: lane 4*s + q (< 32) holds the source row of contraction row q of this wave in step s of the burst
+  int l_g_lo = 0, l_g_nk = 0;
+  const uint32_t g_row_bytes = uint32_t((kGatherB ? p.ldb : p.lda) * 2);
+  constexpr int kGatherBurst = 8;  // wgrad: steps served by one round of scalar loads
+  // (src_rows is padded past its last row -- 512 entries, stm_row_sources_padding() -- so that
+  // none of the scalar loads below needs a bounds check: a rows-form tile reaches at most 255
+  // rows past the end, a wgrad burst at most 31 + 8 * kBK; what they read there belongs to rows
+  // that are dropped)
+  auto uniform_ptr = [](const int32_t* q) {  // the same pointer, provably wave-uniform
+    const uint64_t v = reinterpret_cast<uint64_t>(q);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(uint32_t(v)), hi = __builtin_amdgcn_readfirstlane(uint32_t(v >> 32));
+    return reinterpret_cast<const int32_t*>((uint64_t(hi) << 32) | lo);
+  };
+  auto gather_rows_of_tile = [&]() {  // rows form: tile rows wave*32 .. +31 are this wave's to load
+    if constexpr (kGatherA && !WGRAD) {
+      int mine = 0;  // lane i < 32: source row of tile row wave*32 + i
+      const int32_t* from = uniform_ptr(p.src_rows + (int64_t(l_g_lo) + wave * 32));
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        const int value = __builtin_amdgcn_readfirstlane(scalar_load(from, i));
+        asm("v_writelane_b32 %0, %1, %2" : "+v"(mine) : "s"(value), "n"(i));
+      }
+#pragma unroll
+      for (int j = 0; j < kLoadsA; ++j) {
+        const int rel = j * PlanA::kRowsPerLoad + plan_a.row_in_load;
+        const int src = __builtin_amdgcn_ds_bpermute(rel * 4, mine);
+        g_voff[j] = wave * 32 + rel < l_g_nk ? uint32_t(src) * g_row_bytes + plan_a.col[j & 1] : kGatherDropped;
+      }
+    }
+  };
+  // wgrad: a wave loads contraction rows step*kBK + wave*4 .. +3 of the group in every step
+  auto gather_fetch_burst = [&](int step0) {
+    if constexpr (GATHER != 0 && WGRAD) {
+      const int32_t* from = uniform_ptr(p.src_rows + (int64_t(l_g_lo) + int64_t(step0) * kBK + wave * 4));
+#pragma unroll
+      for (int i = 0; i < kGatherBurst * 4; ++i) {
+        const int value = __builtin_amdgcn_readfirstlane(scalar_load(from, (i / 4) * kBK + i % 4));
+        asm("v_writelane_b32 %0, %1, %2" : "+v"(g_bank) : "s"(value), "n"(i));
+      }
+    }
+  };
+  // The lanes fetch their source rows from the bank here, when the cursor enters the step; the
+  // lane offsets are formed from them only when the loads are issued, most of a step later, so
+  // that nothing waits for the cross-lane read.
+  int g_limit = 0;  // contraction rows of the group left at this wave's first row of the step
+  auto gather_apply_step = [&](int step) {
+    if constexpr (GATHER != 0 && WGRAD) {
+      const int ril = kGatherB ? plan_b.row_in_load : plan_a.row_in_load;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        g_voff[j] = uint32_t(__builtin_amdgcn_ds_bpermute(((step % kGatherBurst) * 4 + j * 2 + ril) * 4, g_bank));
+      g_limit = __builtin_amdgcn_readfirstlane(l_g_nk - (step * kBK + wave * 4));
+    }
+  };
+  auto gathered_offset = [&](int j) -> uint32_t {
+    if constexpr (GATHER != 0 && WGRAD) {
+      const int ril = kGatherB ? plan_b.row_in_load : plan_a.row_in_load;
+      const uint32_t col = kGatherB ? plan_b.col[j & 1] : plan_a.col[j & 1];
+      return j * 2 + ril < g_limit ? g_voff[j] * g_row_bytes + col : kGatherDropped;
+    } else {
+      return g_voff[j];
+    }
+  };
+  const uint32_t l_soff_a0 = kGatherA ? 0u : plan_a.stage_soffset(0, wave);
   uint32_t l_soff_b0 = plan_b.stage_soffset(0, wave);  // per tile for the fused forward
   const uint32_t l_lds_a0 = __builtin_amdgcn_readfirstlane(lds_base + uint32_t(wave * kLoadsA) * 1024u);
   const uint32_t l_lds_b0 =
@@ -464,12 +574,31 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
     if constexpr (EPI == kSwigluFwd) l_soff_b0 = __builtin_amdgcn_readfirstlane(t.soff_b0);
     l_soff_a = l_soff_a0;
     l_soff_b = l_soff_b0;
+    if constexpr (GATHER != 0) {
+      l_g_lo = __builtin_amdgcn_readfirstlane(t.g_lo);
+      l_g_nk = __builtin_amdgcn_readfirstlane(t.g_nk);
+      if constexpr (WGRAD) {  // the column offset is the scalar offset, the row sits in the lane offset
+        if constexpr (kGatherA) l_soff_a = __builtin_amdgcn_readfirstlane(t.g_soff);
+        if constexpr (kGatherB) l_soff_b = __builtin_amdgcn_readfirstlane(t.g_soff);
+        gather_fetch_burst(0);
+        gather_apply_step(0);
+      } else {
+        gather_rows_of_tile();
+      }
+    }
   };
   auto issue_one_load = [&](int li) {  // li is a compile-time constant at every call site
-    if (li < kLoadsA)
-      plan_a.issue_one(l_rsrc_a, l_lds_a0 + l_slot, l_soff_a, li);
-    else
-      plan_b.issue_one(l_rsrc_b, l_lds_b0 + l_slot, l_soff_b, li - kLoadsA);
+    if (li < kLoadsA) {
+      if constexpr (kGatherA)
+        plan_a.issue_gathered(l_rsrc_a, l_lds_a0 + l_slot, l_soff_a, li, gathered_offset(li));
+      else
+        plan_a.issue_one(l_rsrc_a, l_lds_a0 + l_slot, l_soff_a, li);
+    } else {
+      if constexpr (kGatherB)
+        plan_b.issue_gathered(l_rsrc_b, l_lds_b0 + l_slot, l_soff_b, li - kLoadsA, gathered_offset(li - kLoadsA));
+      else
+        plan_b.issue_one(l_rsrc_b, l_lds_b0 + l_slot, l_soff_b, li - kLoadsA);
+    }
   };
   auto issue_loads = [&](auto first_tag, auto last_tag) {
     constexpr int kFirst = decltype(first_tag)::value, kLast = decltype(last_tag)::value;
@@ -478,11 +607,13 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
   };
   auto advance_loads = [&]() {  // the stage under the cursor is fully issued: move to the next
     l_slot = (l_slot + kStageBytes) & (kStages * kStageBytes - 1);
-    l_soff_a += plan_a.step_bytes;
-    l_soff_b += plan_b.step_bytes;
-    if (++l_step >= l_n_steps) {
-      l_k += wgs_per_xcd;
-      const int id = tile_id(l_k);
+    if constexpr (!(kGatherA && WGRAD)) l_soff_a += plan_a.step_bytes;
+    if constexpr (!(kGatherB && WGRAD)) l_soff_b += plan_b.step_bytes;
+    // (pinned: everything the cursor decides on is wave-uniform and must stay on the scalar unit)
+    l_step = __builtin_amdgcn_readfirstlane(l_step + 1);
+    if (__builtin_amdgcn_readfirstlane(int(l_step >= l_n_steps))) {
+      l_k = __builtin_amdgcn_readfirstlane(l_k + wgs_per_xcd);
+      const int id = __builtin_amdgcn_readfirstlane(tile_id(l_k));
       TileState<T> t;
       if (id >= 0) {
         locate(id, t);
@@ -490,8 +621,13 @@ __global__ __launch_bounds__(WAVES* kWave) void persistent_gemm_kernel(GemmArgs 
         t.rsrc_a = make_rsrc(p.a, 0);
         t.rsrc_b = make_rsrc(p.b, 0);
         t.n_steps = 0x7fffffff;
+        t.g_lo = t.g_nk = 0;
+        t.g_soff = 0;
       }
       load_tile(t);
+    } else if constexpr (GATHER != 0 && WGRAD) {
+      if (l_step % kGatherBurst == 0) gather_fetch_burst(l_step);
+      gather_apply_step(l_step);
     }
   };
 
@@ -1060,9 +1196,9 @@ int persistent_grid() {
   return cached;
 }
 
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int BK, int EPI, bool PP>
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int WAVES, int BK, int EPI, bool PP, int GATHER>
 int launch_waves(const GemmArgs& p, hipStream_t s) {
-  auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD, WAVES, BK, EPI, PP>;
+  auto kernel = persistent_gemm_kernel<T, BM, BN, A_KM, B_KM, WGRAD, WAVES, BK, EPI, PP, GATHER>;
   constexpr size_t smem = (size_t(1) << kStagesBytesLog2) + size_t(kEpilogueBytes);
   static bool configured = false;
   if (!configured) {
@@ -1093,13 +1229,18 @@ bool use_pingpong(Product which) {
   return which == kWgrad;
 }
 
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int BK, int EPI = kStore>
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int BK, int EPI = kStore, int GATHER = 0>
 int launch(const GemmArgs& p, hipStream_t s) {
-  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, kGemmWaves, BK, EPI, false>(p, s);
+  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, kGemmWaves, BK, EPI, false, GATHER>(p, s);
 }
-template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int EPI = kStore>
+template <typename T, int BM, int BN, bool A_KM, bool B_KM, bool WGRAD, int EPI = kStore, int GATHER = 0>
 int launch_pp(const GemmArgs& p, hipStream_t s) {
-  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, kGemmWaves, 32, EPI, true>(p, s);
+  return launch_waves<T, BM, BN, A_KM, B_KM, WGRAD, kGemmWaves, 32, EPI, true, GATHER>(p, s);
+}
+
+// A gathered operand: the table and a buffer small enough for 31-bit lane offsets.
+bool gather_ok(const GemmArgs& p) {
+  return p.src_rows != nullptr && p.src_n_rows > 0 && p.src_bytes > 0 && p.src_bytes < 0x80000000u;
 }
 
 }  // namespace
@@ -1158,6 +1299,11 @@ int launch_dma_swiglu_fwd(int dtype, const GemmArgs& base, const int32_t* offset
   if (st != STM_OK) return st;
   p.tiles_j = (p.ffn + kDmaBN / 2 - 1) / (kDmaBN / 2);
   if (!prepare_tile_ids(p, max_m_tiles(m_cap, n_groups, kDmaBM))) return STM_ERR_UNSUPPORTED;
+  if (p.src_rows) {  // (one schedule: the product's default)
+    if (!gather_ok(p) || p.n_k % 64 != 0) return STM_ERR_UNSUPPORTED;
+    if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, false, false, false, 64, kSwigluFwd, 1>(p, s);
+    return launch<f16_t, kDmaBM, kDmaBN, false, false, false, 64, kSwigluFwd, 1>(p, s);
+  }
   if (use_pingpong(kFusedFwd)) {
     if (dtype == STM_BF16) return launch_pp<bf16_t, kDmaBM, kDmaBN, false, false, false, kSwigluFwd>(p, s);
     return launch_pp<f16_t, kDmaBM, kDmaBN, false, false, false, kSwigluFwd>(p, s);
@@ -1183,6 +1329,11 @@ int launch_dma_swiglu_bwd(int dtype, const GemmArgs& base, const int32_t* offset
   p.n_j = p.ffn;
   p.tiles_j = (p.ffn + kDmaBN - 1) / kDmaBN;
   if (!prepare_tile_ids(p, max_m_tiles(m_cap, n_groups, kDmaBM))) return STM_ERR_UNSUPPORTED;
+  if (p.src_rows) {
+    if (!gather_ok(p)) return STM_ERR_UNSUPPORTED;
+    if (dtype == STM_BF16) return launch<bf16_t, kDmaBM, kDmaBN, false, true, false, 32, kSwigluBwd, 1>(p, s);
+    return launch<f16_t, kDmaBM, kDmaBN, false, true, false, 32, kSwigluBwd, 1>(p, s);
+  }
   if (use_pingpong(kFusedBwd)) {
     if (dtype == STM_BF16) return launch_pp<bf16_t, kDmaBM, kDmaBN, false, true, false, kSwigluBwd>(p, s);
     return launch_pp<f16_t, kDmaBM, kDmaBN, false, true, false, kSwigluBwd>(p, s);
@@ -1221,6 +1372,15 @@ int launch_dma_wgrad(int dtype, const GemmArgs& base, int n_groups, int64_t m_ca
   p.tiles_j = (p.n_j + kDmaBN - 1) / kDmaBN;
   p.n_groups = n_groups;
   if (!prepare_tile_ids(p, int64_t(n_groups) * p.tiles_i)) return STM_ERR_UNSUPPORTED;
+  if (p.src_rows) {
+    if (!gather_ok(p) || accumulate || (p.gather_operand != 1 && p.gather_operand != 2)) return STM_ERR_UNSUPPORTED;
+    if (p.gather_operand == 1) {
+      if (dtype == STM_BF16) return launch_pp<bf16_t, kDmaBM, kDmaBN, true, true, true, kStore, 1>(p, s);
+      return launch_pp<f16_t, kDmaBM, kDmaBN, true, true, true, kStore, 1>(p, s);
+    }
+    if (dtype == STM_BF16) return launch_pp<bf16_t, kDmaBM, kDmaBN, true, true, true, kStore, 2>(p, s);
+    return launch_pp<f16_t, kDmaBM, kDmaBN, true, true, true, kStore, 2>(p, s);
+  }
   if (use_pingpong(kWgrad)) {
     if (accumulate) {
       if (dtype == STM_BF16) return launch_pp<bf16_t, kDmaBM, kDmaBN, true, true, true, kAccumF32>(p, s);

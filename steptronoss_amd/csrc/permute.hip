@@ -352,6 +352,15 @@ __global__ void slot_values_to_rows_kernel(const W* __restrict__ values, const i
   if (r >= 0 && r < n_rows) rows[r] = to_float(values[s]);
 }
 
+// token_of_row[pos[s]] = s / top_k: the token whose copy row pos[s] of the permuted order would be.
+__global__ void slot_tokens_to_rows_kernel(const int32_t* __restrict__ pos, int64_t n_slots, int top_k,
+                                           int32_t* __restrict__ token_of_row, int64_t n_rows) {
+  const int64_t s = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (s >= n_slots) return;
+  const int64_t r = pos[s];
+  if (r >= 0 && r < n_rows) token_of_row[r] = int32_t(s / top_k);
+}
+
 // out[s] = sum of the n_parts numbers of row pos[s].
 template <typename W>
 __global__ void row_parts_to_slots_kernel(const float* __restrict__ parts, int n_parts, const int32_t* __restrict__ pos,
@@ -864,6 +873,17 @@ int stm_slot_values_to_rows(const void* values, int value_dtype, const int32_t* 
     case STM_BF16: slot_values_to_rows_kernel<<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(values), pos, n_slots, rows, n_rows); break;
     default: return STM_ERR_UNSUPPORTED;
   }
+  return launch_status();
+}
+
+int stm_slot_tokens_to_rows(const int32_t* pos, int64_t n_slots, int top_k, int32_t* token_of_row, int64_t n_rows,
+                            stm_stream_t stream) {
+  using namespace stm;
+  if (n_slots < 0 || n_rows < 0 || top_k <= 0 || n_slots / top_k > 0x7fffffff) return STM_ERR_ARG;
+  if (n_slots == 0 || n_rows == 0) return STM_OK;
+  if (!pos || !token_of_row) return STM_ERR_ARG;
+  slot_tokens_to_rows_kernel<<<unsigned((n_slots + 255) / 256), 256, 0, as_stream(stream)>>>(pos, n_slots, top_k,
+                                                                                            token_of_row, n_rows);
   return launch_status();
 }
 

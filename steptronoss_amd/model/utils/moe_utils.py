@@ -69,6 +69,11 @@ class Settings:
         (bf16 / fp16 inputs, hidden a multiple of 64, at most 512 experts): the logits never reach
         HBM and no fp32 copies of the inputs are made.  ``"always"``: 16-bit gate outputs as well
         (there library GEMM + router is the faster pair).  Off: ``MoEGate`` then the router.
+    gather_in_gemm: the fused ``routed_grouped_ffn`` (bf16 / fp16, ``x`` below 2 GiB) makes no
+        permuted copy of ``x`` (reference ``moe_scatter``, moe_utils.py:226) nor of ``grad_out``: the
+        GEMMs that read those rows (forward 1, both weight gradients, the input gradient of GEMM 2)
+        gather them through a row -> token table in their loads.  Off, or for a shape those kernels
+        do not take: the rows are copied first, as before.
     deferred_id_check: ``routed_grouped_ffn`` copies the routing status words to pinned host
         memory without waiting; a later call (or ``check_deferred_status()``) that finds such a
         copy complete raises the reference's "out-of-range" ``ValueError`` for an expert id
@@ -83,6 +88,7 @@ class Settings:
     deferred_id_check: bool = True
     fp8_experts: bool = False
     fuse_gate: bool | str = True
+    gather_in_gemm: bool = True
 
 
 settings = Settings()
@@ -637,6 +643,86 @@ def _gemm_dswiglu_rows(gy, w2, gu, offsets, swiglu_limit, row_scale=None, row_do
     return dgu if ok else None
 
 
+def _permuted_rows(x: torch.Tensor, pos: torch.Tensor, top_k: int) -> torch.Tensor:
+    """``out[pos[t, k]] = x[t]``: the copy of the token rows in expert order (all ``T*K`` rows)."""
+    n_tokens, hidden = x.shape
+    n_rows = n_tokens * top_k
+    out = torch.empty((n_rows, hidden), device=x.device, dtype=x.dtype)
+    call(
+        "stm_permute_fwd", ptr(x), ptr(pos), 0, ptr(out), n_tokens, top_k, hidden * x.element_size(), n_rows, None,
+        stream(),
+    )  # fmt: skip
+    return out
+
+
+def _takes_main_grad(weight: torch.Tensor) -> bool:
+    """Whether the weight gradient goes into ``weight.main_grad`` (which reads copied rows)."""
+    return settings.fuse_main_grad and getattr(weight, "main_grad", None) is not None
+
+
+def _token_of_row(pos: torch.Tensor, top_k: int) -> torch.Tensor:
+    """int32 ``[T*K (+ padding)]``: the token whose copy row ``r`` of the permuted order would be.
+    Entries of unused rows and of the padding (``stm_row_sources_padding()`` entries, which let
+    the kernels fetch the table in blocks without bounds checks) keep whatever the buffer held:
+    they only ever address rows that are dropped."""
+    n_rows = pos.numel()
+    out = torch.empty(n_rows + int(_lib.load().stm_row_sources_padding()), device=pos.device, dtype=torch.int32)
+    call("stm_slot_tokens_to_rows", ptr(pos), n_rows, top_k, ptr(out), n_rows, stream())
+    return out[:n_rows]
+
+
+def _gathered_takes(src: torch.Tensor) -> bool:
+    """A tensor the GEMM loads can gather rows from: 16-bit, contiguous, below 2 GiB."""
+    return (
+        settings.gather_in_gemm and src.dtype in (torch.bfloat16, torch.float16) and src.is_contiguous()
+        and 0 < src.numel() * src.element_size() < 2**31
+    )  # fmt: skip
+
+
+def _gemm_swiglu_rows_gathered(x, token_of_row, w1, offsets, swiglu_limit, row_scale=None):
+    """:func:`_gemm_swiglu_rows` on the rows ``x[token_of_row]`` without copying them first."""
+    m_cap, k = token_of_row.numel(), x.shape[1]
+    n_groups, two_f, _ = w1.shape
+    ffn = two_f // 2
+    gu = torch.empty((m_cap, two_f), device=x.device, dtype=x.dtype)
+    h = torch.empty((m_cap, ffn), device=x.device, dtype=x.dtype)
+    ws = _gemm_workspace(m_cap, n_groups, x.device)
+    ok = try_call(
+        "stm_grouped_gemm_swiglu_gathered", ptr(x), x.shape[0], ptr(token_of_row), ptr(w1), ptr(gu), ptr(h), ptr(row_scale),
+        ptr(offsets), n_groups, m_cap, ffn, k, int(swiglu_limit is not None), float(swiglu_limit or 0.0),
+        dtype_code(x.dtype), ptr(ws), ws.numel(), stream(),
+    )  # fmt: skip
+    return (gu, h) if ok else (None, None)
+
+
+def _gemm_dswiglu_rows_gathered(go, token_of_row, w2, gu, offsets, swiglu_limit, row_scale=None, row_dot=None):
+    """:func:`_gemm_dswiglu_rows` on the rows ``go[token_of_row]`` without copying them first."""
+    m_cap, k = token_of_row.numel(), go.shape[1]
+    n_groups, _, ffn = w2.shape
+    dgu = torch.empty_like(gu)
+    ws = _gemm_workspace(m_cap, n_groups, go.device)
+    ok = try_call(
+        "stm_grouped_gemm_dswiglu_gathered", ptr(go), go.shape[0], ptr(token_of_row), ptr(w2), ptr(gu), ptr(dgu),
+        ptr(row_scale), ptr(row_dot), ptr(offsets), n_groups, m_cap, ffn, k, int(swiglu_limit is not None),
+        float(swiglu_limit or 0.0), dtype_code(go.dtype), ptr(ws), ws.numel(), stream(),
+    )  # fmt: skip
+    return dgu if ok else None
+
+
+def _gemm_wgrad_gathered(x, y, offsets, n_groups, token_of_row, gathered_operand: int):
+    """:func:`_gemm_wgrad` with ``x`` (operand 1) or ``y`` (operand 2) standing for its rows
+    ``[token_of_row]``; ``None`` when the kernel does not take the shape."""
+    m_cap = token_of_row.numel()
+    p, q = x.shape[1], y.shape[1]
+    out = torch.empty((n_groups, p, q), device=x.device, dtype=x.dtype)
+    src = x if gathered_operand == 1 else y
+    ok = try_call(
+        "stm_grouped_gemm_wgrad_gathered", ptr(x), ptr(y), ptr(out), ptr(offsets), n_groups, m_cap, p, q,
+        dtype_code(x.dtype), ptr(token_of_row), gathered_operand, src.shape[0], stream(),
+    )  # fmt: skip
+    return out if ok else None
+
+
 def _wgrad_into_main_grad(x: torch.Tensor, y: torch.Tensor, offsets: torch.Tensor, weight: torch.Tensor) -> bool:
     """``weight.main_grad[g] += x[rows of g]^T @ y[rows of g]`` when the switch is on, the
     buffer is there (fp32, the weight's shape) and the kernel takes the shape."""
@@ -697,10 +783,6 @@ class _FusedRoutedFFN(torch.autograd.Function):
             elif settings.deferred_id_check:
                 _defer_status_check(status)
             live = offsets[E:]  # device word: number of used rows
-            xp = torch.empty((n_rows, H), device=dev, dtype=x.dtype)
-            call(
-                "stm_permute_fwd", ptr(x), ptr(pos), 0, ptr(xp), T, K, H * x.element_size(), n_rows, None, stream()
-            )
             w_row = None
             if settings.weights_before_gemm2 and token_weights.dtype == torch.float32:
                 w_row = torch.empty(n_rows, device=dev, dtype=torch.float32)
@@ -708,7 +790,15 @@ class _FusedRoutedFFN(torch.autograd.Function):
                     "stm_slot_values_to_rows", ptr(token_weights), dtype_code(token_weights.dtype), ptr(pos), n_rows,
                     ptr(w_row), n_rows, stream(),
                 )  # fmt: skip
-            gu, h = _gemm_swiglu_rows(xp, w1, offsets, swiglu_limit, w_row)
+            # the first GEMM reads the token rows of x through the row -> token table; the permuted
+            # copy is only made when that kernel does not take the shape
+            xp = token_of_row = gu = h = None
+            if _gathered_takes(x):
+                token_of_row = _token_of_row(pos, K)
+                gu, h = _gemm_swiglu_rows_gathered(x, token_of_row, w1, offsets, swiglu_limit, w_row)
+            if h is None:
+                xp = _permuted_rows(x, pos, K)
+                gu, h = _gemm_swiglu_rows(xp, w1, offsets, swiglu_limit, w_row)
             if h is None:
                 w_row = None
                 gu = _gemm_rows(xp, w1, offsets, two_f, True)
@@ -717,10 +807,10 @@ class _FusedRoutedFFN(torch.autograd.Function):
             addend = None if out_addend is None else out_addend.contiguous()
             if w_row is None:
                 out = _combine_rows(y, pos, token_weights, out_scale, addend)
-                ctx.save_for_backward(w1, w2, x, xp, gu, h, y, pos, offsets, token_weights)
+                ctx.save_for_backward(w1, w2, x, xp, gu, h, y, pos, offsets, token_weights, token_of_row)
             else:  # h and y carry the weights already
                 out = _combine_rows(y, pos, _unit_weights(pos.shape, dev), out_scale, addend)
-                ctx.save_for_backward(w1, w2, x, xp, gu, h, w_row, pos, offsets, token_weights)
+                ctx.save_for_backward(w1, w2, x, xp, gu, h, w_row, pos, offsets, token_weights, token_of_row)
             _nothing_routed_fwd(live, x, token_weights, out, out_scale, addend)
         ctx.weighted_rows = w_row is not None
         ctx.limit = swiglu_limit
@@ -732,7 +822,7 @@ class _FusedRoutedFFN(torch.autograd.Function):
     def backward(ctx, grad_out):
         from steptronoss_amd.model.common.feed_forward import swiglu_bwd_rows, swiglu_fwd_rows
 
-        w1, w2, x, xp, gu, h, y_or_w_row, pos, offsets, token_weights = ctx.saved_tensors
+        w1, w2, x, xp, gu, h, y_or_w_row, pos, offsets, token_weights, token_of_row = ctx.saved_tensors
         T, H, K, E = ctx.shape
         dev = grad_out.device
         need_w1, need_w2, need_x, _, need_tw, _, _, need_addend = ctx.needs_input_grad
@@ -741,20 +831,25 @@ class _FusedRoutedFFN(torch.autograd.Function):
             live = offsets[E:]
             go = go_unscaled = grad_out.contiguous()
             dgu = None
+            gathered = token_of_row is not None
+            gy = None
             if ctx.weighted_rows:
                 w_row = y_or_w_row
-                n_rows = xp.shape[0]
+                n_rows = T * K
                 if ctx.out_scale is not None:
                     go = go * ctx.out_scale
-                gy = torch.empty_like(xp)  # rows of grad_out, one per routed slot
-                call(
-                    "stm_permute_fwd", ptr(go), ptr(pos), 0, ptr(gy), T, K, H * go.element_size(), n_rows, None, stream()
-                )
+                # d y is one row of grad_out per routed slot: gathered by the kernels that read it,
+                # copied out (gy) only for a kernel that does not take the shape
+                gathered_go = gathered and _gathered_takes(go)
                 if need_w1 or need_x or need_tw:
                     ffn = h.shape[1]
                     n_parts = _row_dot_parts(ffn)
                     parts = torch.empty((n_rows, n_parts), device=dev, dtype=torch.float32)
-                    dgu = _gemm_dswiglu_rows(gy, w2, gu, offsets, ctx.limit, w_row, parts)
+                    if gathered_go:
+                        dgu = _gemm_dswiglu_rows_gathered(go, token_of_row, w2, gu, offsets, ctx.limit, w_row, parts)
+                    if dgu is None:
+                        gy = _permuted_rows(go, pos, K)
+                        dgu = _gemm_dswiglu_rows(gy, w2, gu, offsets, ctx.limit, w_row, parts)
                     if dgu is None:  # the fused kernel declined: the same arithmetic, step by step
                         dhu = _gemm_rows(gy, w2, offsets, ffn, False)
                         parts = (swiglu_fwd_rows(gu, ctx.limit, live).float() * dhu.float()).sum(1, keepdim=True)
@@ -766,11 +861,16 @@ class _FusedRoutedFFN(torch.autograd.Function):
                             "stm_row_parts_to_slots", ptr(parts), n_parts, ptr(pos), n_rows, n_rows, ptr(gtw),
                             dtype_code(gtw.dtype), stream(),
                         )  # fmt: skip
+                if need_w2:
+                    if gy is None and gathered_go and not _takes_main_grad(w2):
+                        gw2 = _gemm_wgrad_gathered(go, h, offsets, E, token_of_row, 1)
+                    if gw2 is None and gy is None:
+                        gy = _permuted_rows(go, pos, K)
             else:
                 y = y_or_w_row
                 gy = torch.empty_like(y)
                 gtw = _combine_rows_bwd(go, y, pos, token_weights, gy, None, ctx.out_scale)
-            if need_w2 and not _wgrad_into_main_grad(gy, h, offsets, w2):
+            if need_w2 and gw2 is None and not _wgrad_into_main_grad(gy, h, offsets, w2):
                 gw2 = _gemm_wgrad(gy, h, offsets, E)
             if need_w1 or need_x:
                 if dgu is None:
@@ -778,8 +878,14 @@ class _FusedRoutedFFN(torch.autograd.Function):
                 if dgu is None:
                     dh = _gemm_rows(gy, w2, offsets, h.shape[1], False)
                     dgu = swiglu_bwd_rows(gu, dh, ctx.limit, live)
-                if need_w1 and not _wgrad_into_main_grad(dgu, xp, offsets, w1):
-                    gw1 = _gemm_wgrad(dgu, xp, offsets, E)
+                if need_w1:
+                    if xp is None and not _takes_main_grad(w1):
+                        gw1 = _gemm_wgrad_gathered(dgu, x, offsets, E, token_of_row, 2)
+                    if gw1 is None:
+                        if xp is None:
+                            xp = _permuted_rows(x, pos, K)
+                        if not _wgrad_into_main_grad(dgu, xp, offsets, w1):
+                            gw1 = _gemm_wgrad(dgu, xp, offsets, E)
                 if need_x:
                     dxp = _gemm_rows(dgu, w1, offsets, H, False)
                     gx = _permute_rows_bwd(dxp, pos, H)

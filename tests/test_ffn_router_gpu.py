@@ -160,7 +160,8 @@ def test_ffn_on_the_fused_kernels_with_weights_at_either_place(weights_before_ge
     with KernelTimer() as kt:
         _ffn_case(1024, 128, 8, 16, Fh, dtype, "own", inv, BF16_TOL, seed=3, limit=limit, std=0.3)
     ran = set(kt.summary())
-    assert {"stm_grouped_gemm_swiglu", "stm_grouped_gemm_dswiglu"} <= ran
+    assert ran & {"stm_grouped_gemm_swiglu", "stm_grouped_gemm_swiglu_gathered"}
+    assert ran & {"stm_grouped_gemm_dswiglu", "stm_grouped_gemm_dswiglu_gathered"}
     if weights_before_gemm2:
         assert {"stm_slot_values_to_rows", "stm_row_parts_to_slots"} <= ran and "stm_unpermute_bwd_scaled" not in ran
     else:
@@ -233,12 +234,58 @@ def test_ffn_backward_when_the_fused_dgrad_declines(monkeypatch):
         return [t.grad for t in ins]
 
     fused = run()
-    real = M._gemm_dswiglu_rows
-    monkeypatch.setattr(M, "_gemm_dswiglu_rows", lambda *a, **k: None)
-    stepwise = run()
-    monkeypatch.setattr(M, "_gemm_dswiglu_rows", real)
+    with monkeypatch.context() as mp:
+        mp.setattr(M, "_gemm_dswiglu_rows", lambda *a, **k: None)
+        mp.setattr(M, "_gemm_dswiglu_rows_gathered", lambda *a, **k: None)
+        stepwise = run()
     for a, b in zip(fused, stepwise):
         assert rel_l2(a, b.float()) <= 5e-3
+
+
+@pytest.mark.parametrize("weights_before_gemm2", [True, False], indirect=True)
+@pytest.mark.parametrize("dtype,inv,E,T", [(torch.bfloat16, 0.15, 8, 2048), (torch.float16, 0.0, 8, 2048), (torch.bfloat16, 0.3, 24, 3001)])
+def test_ffn_gathers_token_rows_in_the_gemm_loads(weights_before_gemm2, dtype, inv, E, T):
+    # The permuted copies of x (moe_scatter, reference moe_utils.py:226) and of grad_out are not
+    # made: forward 1, the input gradient of GEMM 2 and both weight gradients read the token rows
+    # through a row -> token table.  Same loads, same arithmetic: identical bits to the copying path.
+    from steptronoss_amd.profiling import KernelTimer
+
+    gen = torch.Generator().manual_seed(21)
+    H, K, Fh = 512, 4, 256
+    x = (torch.randn(T, H, generator=gen) * 0.5).to(dtype)
+    w1 = (torch.randn(E, 2 * Fh, H, generator=gen) * 0.05).to(dtype)
+    w2 = (torch.randn(E, H, Fh, generator=gen) * 0.05).to(dtype)
+    ids = make_topk_ids(T, K, E, gen=gen, invalid_frac=inv)
+    ids = torch.where(ids == 3, torch.full_like(ids, -1), ids).to(DEV)  # an expert without tokens
+    tw = torch.rand(T, K, generator=gen)
+    go = torch.randn(T, H, generator=gen).to(dtype).to(DEV)
+
+    def run(gather):
+        old = M.settings.gather_in_gemm
+        M.settings.gather_in_gemm = gather
+        try:
+            ins = [t.to(DEV).requires_grad_(True) for t in (w1, w2, x, tw)]
+            with KernelTimer() as kt:
+                out = M.routed_grouped_ffn(ins[0], ins[1], swiglu, ins[2], ids, ins[3])
+                out.backward(go)
+            return [out.detach()] + [t.grad for t in ins], set(kt.summary())
+        finally:
+            M.settings.gather_in_gemm = old
+
+    gathered, ran = run(True)
+    copied, ran_copied = run(False)
+    assert "stm_permute_fwd" in ran_copied and "stm_grouped_gemm_swiglu_gathered" not in ran_copied
+    assert "stm_permute_fwd" not in ran
+    assert {"stm_slot_tokens_to_rows", "stm_grouped_gemm_swiglu_gathered", "stm_grouped_gemm_wgrad_gathered"} <= ran
+    assert ("stm_grouped_gemm_dswiglu_gathered" in ran) == weights_before_gemm2
+    for name, a, b in zip(("out", "dw1", "dw2", "dx", "dtw"), gathered, copied):
+        assert torch.equal(a, b), name
+    ref_in = [t.clone().float().requires_grad_(True) for t in (w1, w2, x, tw)]
+    ref = O.routed_grouped_ffn(ref_in[0], ref_in[1], O.swiglu, ref_in[2], ids.cpu(), ref_in[3])
+    ref.backward(go.cpu().float())
+    assert rel_l2(gathered[0], ref) <= BF16_TOL
+    for got, r in zip(gathered[1:], ref_in):
+        assert rel_l2(got, r.grad) <= BF16_TOL
 
 
 def test_slot_and_row_order_helpers():
