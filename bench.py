@@ -41,9 +41,9 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 # --traffic-probe).  Each figure names the summary under profiles/ it was taken from and holds
 # for the kernels of that summary only: None = not measured for the kernels as they are now.
 MEASURED_GEMM_TRAFFIC = {
-    "c2": {"bytes": None, "source": "profiles/persistent_gemm_c2_hbm_traffic.txt"},
+    "c2": {"bytes": 2.324e9, "source": "profiles/persistent_gemm_c2_hbm_traffic.txt"},
     "c3": {"bytes": None, "source": None},
-    "c4": {"bytes": None, "source": None},
+    "c4": {"bytes": 1.793e10, "source": "profiles/persistent_gemm_c4_hbm_traffic.txt"},
 }
 
 WORKLOADS = {
@@ -100,6 +100,12 @@ def cpu_baseline(cfg, seed, threads):
     torch.set_num_threads(threads)
     T = cfg["T"] // 16
     H, E, F, K = cfg["H"], cfg["E"], cfg["F"], cfg["K"]
+    # fp32 expert weights above 4 GB (the large-expert workload: 45 GB): a subset of the experts,
+    # a multiple of the router's group count, which also keeps the rows per expert near the workload's
+    per_expert = 3 * F * H * 4
+    if E * per_expert > 4e9:
+        unit = max(cfg["n_group"], 1)
+        E = max(2 * unit if unit > 1 else K, int(4e9 // per_expert) // unit * unit)
     gen = torch.Generator().manual_seed(seed)
     x = (torch.randn(T, H, generator=gen) * cfg["std"]).bfloat16().float().requires_grad_(True)
     w1 = (torch.randn(E, 2 * F, H, generator=gen) * cfg["std"]).bfloat16().float().requires_grad_(True)
@@ -126,7 +132,7 @@ def cpu_baseline(cfg, seed, threads):
         "cores": threads,
         "host_cores": os.cpu_count(),
         "kind": "port",
-        "sample": f"{T} of {cfg['T']} tokens over all {E} experts, fp32, fwd+bwd, 1 warm-up + {len(timed)} timed passes "
+        "sample": f"{T} of {cfg['T']} tokens over {E} of {cfg['E']} experts, fp32, fwd+bwd, 1 warm-up + {len(timed)} timed passes "
         f"(mean {mean * 1e3:.0f} ms, warm-up {times[0] * 1e3:.0f} ms) on {threads} threads of {os.cpu_count()} host cores",
     }
 
@@ -242,6 +248,11 @@ def run_fp8(args, cfg):
     print(json.dumps(result))
 
 
+def _progress(msg):
+    """A line on stderr (stdout carries the one JSON line): long workloads show where they are."""
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -274,6 +285,7 @@ def main():
         return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    _progress(f"workload {args.workload}: making inputs")
     x, w1, w2, logits, go = make_inputs(cfg, args.seed, dev)
     for t in (x, w1, w2, logits):
         t.requires_grad_(True)
@@ -291,9 +303,10 @@ def main():
         out = hip_routed_grouped_ffn(w1, w2, swiglu, x, ids, weights)
         torch.autograd.backward([out, aux], [go, one * 0.01])
 
-    for _ in range(args.warmup):
+    for i in range(args.warmup):
         step()
-    torch.cuda.synchronize()
+        torch.cuda.synchronize()
+        _progress(f"warm-up step {i + 1} of {args.warmup} done")
     if args.traffic_probe:
         src = torch.empty(1 << 28, device=dev, dtype=torch.float32).normal_()
         dst = torch.empty_like(src)
@@ -308,6 +321,7 @@ def main():
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
+    _progress(f"{args.steps} timed steps done, {ms_per_step:.3f} ms per step")
     flops = 6.0 * N * H * 3 * F
     value = flops / (ms_per_step * 1e-3) / 1e12
 
@@ -315,7 +329,10 @@ def main():
     fp32 = cfg.get("dtype") == "fp32"
     e = 4 if fp32 else 2  # bytes per element
     peak = PEAK_FP32_TFLOPS if fp32 else PEAK_BF16_TFLOPS
-    gemm_entries = ("stm_grouped_gemm", "stm_grouped_gemm_wgrad", "stm_grouped_gemm_swiglu", "stm_grouped_gemm_dswiglu")
+    gemm_entries = (
+        "stm_grouped_gemm", "stm_grouped_gemm_wgrad", "stm_grouped_gemm_swiglu", "stm_grouped_gemm_dswiglu",
+        "stm_grouped_gemm_wgrad_gathered", "stm_grouped_gemm_swiglu_gathered", "stm_grouped_gemm_dswiglu_gathered",
+    )  # fmt: skip
     gemm_calls = sum(timing[n]["calls"] for n in gemm_entries if n in timing)
     gemm_ms = sum(timing[n]["total_ms"] for n in gemm_entries if n in timing)
     # six equal-cost-per-flop launches per step: 4 over [N, H] x 2F-sized problems count double
@@ -363,7 +380,7 @@ def main():
     })  # fmt: skip
 
     # The stand-alone combine op (moe_weighted_gather, weights applied in the combine), outside
-    # the timed steps: the fused FFN's backward replaces its backward kernel by a row copy.
+    # the timed steps (the fused FFN applies the weights before GEMM 2 and gathers grad_out rows in its GEMM loads).
     from steptronoss_amd.model.utils.moe_utils import histogram, index_compute, moe_weighted_gather
 
     with torch.no_grad():
@@ -374,13 +391,19 @@ def main():
     pos = index_compute(ids, histogram(ids, E))
     rows = torch.randn(N, H, device=dev, dtype=x.dtype).requires_grad_(True)
     slot_weights = weights.detach().clone().requires_grad_(True)
+    from steptronoss_amd.model.utils.moe_utils import moe_scatter
+
+    x_op = x.detach().clone().requires_grad_(True)
     with KernelTimer() as kt_op:
         for _ in range(5):
             rows.grad = slot_weights.grad = None
             moe_weighted_gather(rows, pos, slot_weights).backward(go)
+        for _ in range(5):  # the stand-alone permute (the fused FFN gathers in its GEMM loads instead)
+            x_op.grad = None
+            moe_scatter(x_op, pos).backward(rows.detach())
     for name, t in kt_op.summary().items():
         timing.setdefault(name, t)
-    del rows, slot_weights
+    del rows, slot_weights, x_op
 
     # The gate GEMM folded into the router (outside the timed steps, which start from ready-made
     # logits as the workload is defined): one kernel against library GEMM + router.
@@ -456,6 +479,7 @@ def main():
     }
     if not args.no_cpu_baseline:
         threads = min(os.cpu_count() or 1, 16)  # the box's CPU share is 16 cores whatever the host shows
+        _progress("CPU baseline (the oracle on a sample of the workload)")
         result["cpu_baseline"] = cpu_baseline(cfg, args.seed, threads)
     print(json.dumps(result))
 
