@@ -384,12 +384,15 @@ size_t stm_router_workspace_bytes(int64_t n_tokens, int n_experts);
  * n_group > 1 adds group-limited selection (not in the reference): experts in n_group
  * contiguous groups, group score = sum of its two best scores, only the topk_group best
  * groups stay eligible.
+ * force_balance != 0 (moe_block.py:249-256, "for debug only"): the selection is replaced by
+ * the round-robin assignment ids[t, k] = (t * top_k + k) % n_experts; weights, counts and aux
+ * follow from those ids as above.
  * ids_out int64 [T,K], weights_out fp32 [T,K], aux_out fp32 [1], hist_out int32 [E],
  * me_out fp32 [E]. */
 int stm_router_fwd(const void* logits, int logits_dtype, const float* bias_or_null, int64_t n_tokens, int n_experts,
                    int top_k, int use_sigmoid, int norm_weights, float eps, int n_group, int topk_group,
-                   int64_t* ids_out, float* weights_out, float* aux_out, int32_t* hist_out, float* me_out,
-                   void* workspace, size_t workspace_bytes, stm_stream_t stream);
+                   int force_balance, int64_t* ids_out, float* weights_out, float* aux_out, int32_t* hist_out,
+                   float* me_out, void* workspace, size_t workspace_bytes, stm_stream_t stream);
 
 /* Backward of forward_router w.r.t. the logits (what autograd derives from
  * moe_block.py:229-292): from grad_weights fp32 [T,K] and grad_aux fp32 [1] (may be null). */
@@ -401,7 +404,7 @@ int stm_router_bwd(const void* logits, int logits_dtype, int64_t n_tokens, int n
  * moe_utils.py:64-82: logits = x @ gate_w^T): x [T, hidden] and gate_w [E, hidden] in bf16 or fp16,
  * fp32 accumulation; the logits live in LDS only.  fp32_logits = 0 rounds them to the element type
  * first, as a 16-bit gate output would be (fp32_output = False); 1 keeps them in fp32
- * (fp32_output = True).  STM_ERR_UNSUPPORTED for fp32 inputs, hidden not a multiple of 16 or more
+ * (fp32_output = True).  STM_ERR_UNSUPPORTED for fp32 inputs, hidden not a multiple of 64 or more
  * than 512 experts: callers then compute the logits themselves and call stm_router_fwd.
  * Workspace as for stm_router_fwd.
  * stm_router_gate_bwd recomputes the logits the same way and writes d logits [T, E] (grad_dtype:
@@ -409,9 +412,9 @@ int stm_router_bwd(const void* logits, int logits_dtype, int64_t n_tokens, int n
  * d gate_w are the two dense products of that matrix with gate_w and x. */
 int stm_router_gate_fwd(const void* x, const void* gate_w, int dtype, int hidden, int fp32_logits,
                         const float* bias_or_null, int64_t n_tokens, int n_experts, int top_k, int use_sigmoid,
-                        int norm_weights, float eps, int n_group, int topk_group, int64_t* ids_out, float* weights_out,
-                        float* aux_out, int32_t* hist_out, float* me_out, void* workspace, size_t workspace_bytes,
-                        stm_stream_t stream);
+                        int norm_weights, float eps, int n_group, int topk_group, int force_balance, int64_t* ids_out,
+                        float* weights_out, float* aux_out, int32_t* hist_out, float* me_out, void* workspace,
+                        size_t workspace_bytes, stm_stream_t stream);
 int stm_router_gate_bwd(const void* x, const void* gate_w, int dtype, int hidden, int fp32_logits, int64_t n_tokens,
                         int n_experts, int top_k, int use_sigmoid, int norm_weights, float eps, const int64_t* ids,
                         const float* grad_weights, const float* grad_aux_or_null, const int32_t* hist,

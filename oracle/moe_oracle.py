@@ -380,6 +380,7 @@ def forward_router(
     balance_bias: torch.Tensor | None = None,
     n_group: int = 1,
     topk_group: int = 1,
+    force_balance: bool = False,
 ):
     """Router of moe_block.py:224-292 (single process: the TP/EP all-reduces of the
     count vector at :278-279 are identities).
@@ -393,6 +394,8 @@ def forward_router(
     * sigmoid: weights and scores are each divided by their row sum (+1e-20 iff a
       bias buffer exists) (:261-268); softmax: weights divided by their row sum iff
       ``norm_expert_weight`` (:269-272)
+    * ``force_balance`` (debug switch, :249-256): the ids become ``arange(T*K) % E`` reshaped to
+      ``[T, K]`` and the weights are gathered for those
     * ``aux = sum(mean(scores, 0) * hist) * E`` with ``hist`` the raw per-expert
       counts, which carries no gradient                                  (:274-292)
     """
@@ -402,6 +405,10 @@ def forward_router(
     choice = prob if balance_bias is None else prob + balance_bias.float().unsqueeze(0)
     choice = group_limited_scores(choice, n_group, topk_group)
     _, ids = _stable_topk(choice, top_k)
+    if force_balance:
+        if top_k > E:
+            raise ValueError("force_balance requires top_k <= num_experts")
+        ids = (torch.arange(T * top_k, dtype=torch.int64) % E).view(T, top_k)
     topk_prob = prob.gather(1, ids)
     eps = 1e-20 if balance_bias is not None else 0.0
     weights = topk_prob

@@ -81,8 +81,8 @@ SIGNATURES = {
     "stm_swiglu_fwd": (I, [P, P, L, L, P, I, F, I, P]),
     "stm_swiglu_bwd": (I, [P, P, P, L, L, P, I, F, I, P]),
     "stm_router_workspace_bytes": (Z, [L, I]),
-    "stm_router_fwd": (I, [P, I, P, L, I, I, I, I, F, I, I, P, P, P, P, P, P, Z, P]),
-    "stm_router_gate_fwd": (I, [P, P, I, I, I, P, L, I, I, I, I, F, I, I, P, P, P, P, P, P, Z, P]),
+    "stm_router_fwd": (I, [P, I, P, L, I, I, I, I, F, I, I, I, P, P, P, P, P, P, Z, P]),
+    "stm_router_gate_fwd": (I, [P, P, I, I, I, P, L, I, I, I, I, F, I, I, I, P, P, P, P, P, P, Z, P]),
     "stm_router_gate_bwd": (I, [P, P, I, I, I, L, I, I, I, I, F, P, P, P, P, P, I, P]),
     "stm_router_bias_update": (I, [P, P, I, F, I, P]),
     "stm_router_bwd": (I, [P, I, L, I, I, I, I, F, P, P, P, P, P, P]),

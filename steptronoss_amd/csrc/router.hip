@@ -27,6 +27,7 @@ struct RouterArgs {
   int use_sigmoid, norm_weights;
   int n_group, topk_group;
   float eps;
+  int force_balance;  // round-robin ids instead of the selection (the reference's debug switch)
 };
 
 __device__ __forceinline__ float load_logit(const void* p, int dtype, int64_t i) {
@@ -153,6 +154,11 @@ __device__ __forceinline__ void route_one(const RouterArgs& a, int64_t t_in, int
         slot = j;
         owner = __builtin_ctzll(holders);
       }
+    }
+    if (a.force_balance) {  // reference moe_block.py:253-254: slot (t, r) goes to expert (t*K + r) % E
+      const int forced = __builtin_amdgcn_readfirstlane(int((t_out * K + r) % E));
+      slot = forced / kWave;
+      owner = forced % kWave;
     }
     if (slot < 0) {  // nothing compares equal (NaN scores): the lowest id not taken yet
 #pragma unroll
@@ -759,11 +765,11 @@ size_t stm_router_workspace_bytes(int64_t n_tokens, int n_experts) {
 
 int stm_router_fwd(const void* logits, int logits_dtype, const float* bias_or_null, int64_t n_tokens, int n_experts,
                    int top_k, int use_sigmoid, int norm_weights, float eps, int n_group, int topk_group,
-                   int64_t* ids_out, float* weights_out, float* aux_out, int32_t* hist_out, float* me_out,
-                   void* workspace, size_t workspace_bytes, stm_stream_t stream) {
+                   int force_balance, int64_t* ids_out, float* weights_out, float* aux_out, int32_t* hist_out,
+                   float* me_out, void* workspace, size_t workspace_bytes, stm_stream_t stream) {
   using namespace stm;
   RouterArgs a{logits, logits_dtype, bias_or_null, n_tokens, n_experts, top_k, use_sigmoid, norm_weights,
-               n_group,  topk_group,  eps};
+               n_group,  topk_group,  eps, force_balance != 0};
   const int st = check_router_args(a);
   if (st != STM_OK) return st;
   if (!aux_out || (n_experts > 0 && (!hist_out || !me_out))) return STM_ERR_ARG;
@@ -800,12 +806,12 @@ int stm_router_bwd(const void* logits, int logits_dtype, int64_t n_tokens, int n
 
 int stm_router_gate_fwd(const void* x, const void* gate_w, int dtype, int hidden, int fp32_logits,
                         const float* bias_or_null, int64_t n_tokens, int n_experts, int top_k, int use_sigmoid,
-                        int norm_weights, float eps, int n_group, int topk_group, int64_t* ids_out, float* weights_out,
-                        float* aux_out, int32_t* hist_out, float* me_out, void* workspace, size_t workspace_bytes,
-                        stm_stream_t stream) {
+                        int norm_weights, float eps, int n_group, int topk_group, int force_balance, int64_t* ids_out,
+                        float* weights_out, float* aux_out, int32_t* hist_out, float* me_out, void* workspace,
+                        size_t workspace_bytes, stm_stream_t stream) {
   using namespace stm;
   RouterArgs a{nullptr, STM_F32, bias_or_null, n_tokens, n_experts, top_k, use_sigmoid, norm_weights,
-               n_group, topk_group,   eps};
+               n_group, topk_group,   eps, force_balance != 0};
   int st = check_router_args(a);
   if (st != STM_OK) return st;
   if (n_tokens > 0 && n_experts > 0 && (!x || !gate_w)) return STM_ERR_ARG;

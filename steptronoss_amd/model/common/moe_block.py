@@ -21,7 +21,7 @@ from steptronoss_amd.model.utils.moe_utils import routed_grouped_ffn, settings
 
 class _Router(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, logits, bias, top_k, use_sigmoid, norm_weights, eps, n_group, topk_group):
+    def forward(ctx, logits, bias, top_k, use_sigmoid, norm_weights, eps, n_group, topk_group, force_balance=False):
         dev = require_gpu(logits, bias)
         x = logits.contiguous()
         T, E = x.shape
@@ -36,8 +36,8 @@ class _Router(torch.autograd.Function):
             b = None if bias is None else bias.to(torch.float32).contiguous()
             call(
                 "stm_router_fwd", ptr(x), dtype_code(x.dtype), ptr(b), T, E, top_k, int(use_sigmoid),
-                int(norm_weights), float(eps), int(n_group), int(topk_group), ptr(ids), ptr(weights), ptr(aux),
-                ptr(hist), ptr(me), ptr(ws), ws.numel(), stream(),
+                int(norm_weights), float(eps), int(n_group), int(topk_group), int(force_balance), ptr(ids), ptr(weights),
+                ptr(aux), ptr(hist), ptr(me), ptr(ws), ws.numel(), stream(),
             )  # fmt: skip
         ctx.save_for_backward(x, ids, hist)
         ctx.cfg = (top_k, use_sigmoid, norm_weights, eps)
@@ -61,7 +61,7 @@ class _Router(torch.autograd.Function):
                 "stm_router_bwd", ptr(x), dtype_code(x.dtype), T, E, top_k, int(use_sigmoid), int(norm_weights),
                 float(eps), ptr(ids), ptr(gw), ptr(ga), ptr(hist), ptr(gl), stream(),
             )  # fmt: skip
-        return gl, None, None, None, None, None, None, None
+        return gl, None, None, None, None, None, None, None, None
 
 
 def forward_router(
@@ -73,6 +73,7 @@ def forward_router(
     balance_bias: torch.Tensor | None = None,
     n_group: int = 1,
     topk_group: int = 1,
+    force_balance: bool = False,
 ):
     """Scores, stable top-k, weights and the load-balance loss from ready logits ``[T, E]``.
 
@@ -81,7 +82,8 @@ def forward_router(
     stable descending sort of the scores (plus ``balance_bias`` for selection only), so ties
     go to the lower expert id; weights are renormalised for sigmoid routing or when
     ``norm_expert_weight``; ``aux = E * sum(mean(scores, 0) * hist)``.  ``n_group > 1`` enables
-    group-limited selection.  Returns ``(ids int64 [T,K], weights fp32 [T,K], aux, hist int32
+    group-limited selection; ``force_balance`` (the reference's debug switch, moe_block.py:249-256)
+    replaces the selection by ``ids[t, k] = (t * top_k + k) % E``.  Returns ``(ids int64 [T,K], weights fp32 [T,K], aux, hist int32
     [E])``; differentiable in ``logits`` through ``weights`` and ``aux``.
     """
     if logits.dim() != 2:
@@ -89,7 +91,9 @@ def forward_router(
     if top_k > logits.shape[1]:
         raise ValueError("top_k must not exceed the number of experts")
     eps = 1e-20 if balance_bias is not None else 0.0
-    return _Router.apply(logits, balance_bias, top_k, use_sigmoid, norm_expert_weight, eps, n_group, topk_group)
+    return _Router.apply(
+        logits, balance_bias, top_k, use_sigmoid, norm_expert_weight, eps, n_group, topk_group, force_balance
+    )
 
 
 class _GateRouter(torch.autograd.Function):
@@ -99,7 +103,7 @@ class _GateRouter(torch.autograd.Function):
     ``d x = d logits @ gate_w`` and ``d gate_w = d logits^T @ x`` as two dense library GEMMs."""
 
     @staticmethod
-    def forward(ctx, x, gate_w, bias, top_k, use_sigmoid, norm_weights, eps, n_group, topk_group, fp32_logits):
+    def forward(ctx, x, gate_w, bias, top_k, use_sigmoid, norm_weights, eps, n_group, topk_group, fp32_logits, force_balance=False):
         dev = require_gpu(x, gate_w, bias)
         xc, wc = x.contiguous(), gate_w.contiguous()
         T, H = xc.shape
@@ -115,7 +119,7 @@ class _GateRouter(torch.autograd.Function):
             b = None if bias is None else bias.to(torch.float32).contiguous()
             call(
                 "stm_router_gate_fwd", ptr(xc), ptr(wc), dtype_code(xc.dtype), H, int(fp32_logits), ptr(b), T, E, top_k,
-                int(use_sigmoid), int(norm_weights), float(eps), int(n_group), int(topk_group), ptr(ids), ptr(weights),
+                int(use_sigmoid), int(norm_weights), float(eps), int(n_group), int(topk_group), int(force_balance), ptr(ids), ptr(weights),
                 ptr(aux), ptr(hist), ptr(me), ptr(ws), ws.numel(), stream(),
             )  # fmt: skip
         ctx.save_for_backward(xc, wc, ids, hist)
@@ -144,7 +148,7 @@ class _GateRouter(torch.autograd.Function):
             )  # fmt: skip
             gx = torch.matmul(gl, gate_w) if ctx.needs_input_grad[0] else None
             gwt = torch.matmul(gl.t(), x) if ctx.needs_input_grad[1] else None
-        return gx, gwt, None, None, None, None, None, None, None, None
+        return gx, gwt, None, None, None, None, None, None, None, None, None
 
 
 def gate_router_takes(x: torch.Tensor, gate_w: torch.Tensor) -> bool:
@@ -166,6 +170,7 @@ def forward_gate_router(
     balance_bias: torch.Tensor | None = None,
     n_group: int = 1,
     topk_group: int = 1,
+    force_balance: bool = False,
 ):
     """``forward_router(MoEGate(x))`` (reference moe_block.py:97-113, 224-292) as one kernel: the
     logits ``x @ gate_weight^T`` (fp32 accumulation; rounded to ``x``'s dtype unless ``fp32_output``)
@@ -174,10 +179,11 @@ def forward_gate_router(
     if top_k > gate_weight.shape[0]:
         raise ValueError("top_k must not exceed the number of experts")
     if not gate_router_takes(x, gate_weight):
-        raise ValueError("forward_gate_router: bf16/fp16 x [T, H] with H a multiple of 16 and at most 512 experts")
+        raise ValueError("forward_gate_router: bf16/fp16 x [T, H] with H a multiple of 64 and at most 512 experts")
     eps = 1e-20 if balance_bias is not None else 0.0
     return _GateRouter.apply(
-        x, gate_weight, balance_bias, top_k, use_sigmoid, norm_expert_weight, eps, n_group, topk_group, fp32_output
+        x, gate_weight, balance_bias, top_k, use_sigmoid, norm_expert_weight, eps, n_group, topk_group, fp32_output,
+        force_balance,
     )
 
 
@@ -255,6 +261,7 @@ class MoEBlock(nn.Module):
         swiglu_limit=None,
         n_group=1,
         topk_group=1,
+        force_balance=False,
         router_bias_update_rate=1e-3,
         device=None,
         dtype=None,
@@ -266,6 +273,7 @@ class MoEBlock(nn.Module):
         self.use_sigmoid_router = use_sigmoid_router
         self.norm_expert_weight = norm_expert_weight
         self.n_group, self.topk_group = n_group, topk_group
+        self.force_balance = force_balance  # reference MoEConfig.force_balance, moe_block.py:78-79
         self.gate = MoEGate(hidden_size, num_experts, fp32_gate_output, device=device, dtype=dtype)
         self.experts = GroupedExperts(num_experts, hidden_size, moe_hidden_size, swiglu_limit, device, dtype)
         # aux-loss-free load balancing (reference moe_block.py:199-215): a selection-only bias per
@@ -290,6 +298,7 @@ class MoEBlock(nn.Module):
             balance_bias=self.router_balance_bias,
             n_group=self.n_group,
             topk_group=self.topk_group,
+            force_balance=self.force_balance,
         )
 
     def forward(self, x: torch.Tensor, logits: torch.Tensor | None = None, shared_out: torch.Tensor | None = None):
@@ -305,7 +314,7 @@ class MoEBlock(nn.Module):
             ids, weights, aux, hist = forward_gate_router(
                 x2, self.gate.weight, self.top_k, fp32_output=self.gate.fp32_output, use_sigmoid=self.use_sigmoid_router,
                 norm_expert_weight=self.norm_expert_weight, balance_bias=self.router_balance_bias, n_group=self.n_group,
-                topk_group=self.topk_group,
+                topk_group=self.topk_group, force_balance=self.force_balance,
             )  # fmt: skip
         else:
             if logits is None:

@@ -411,6 +411,32 @@ def test_router_closed_forms():
     assert ids.tolist() == [list(range(16))] * 3
 
 
+@pytest.mark.parametrize("T,E,K,sig,norm", [(257, 128, 8, False, True), (100, 10, 3, True, True), (64, 288, 6, False, False)])
+def test_router_force_balance_matches_reference_rule(T, E, K, sig, norm):
+    # reference moe_block.py:249-256 (debug switch): ids = arange(T*K) % E, weights gathered for them
+    gen = torch.Generator().manual_seed(5)
+    logits = torch.randn(T, E, generator=gen)
+    lr = logits.clone().requires_grad_(True)
+    ref_ids, ref_w, ref_aux, ref_hist = O.forward_router(lr, K, use_sigmoid=sig, norm_expert_weight=norm, force_balance=True)
+    assert torch.equal(ref_ids, (torch.arange(T * K) % E).view(T, K))
+    lg = logits.to(DEV).requires_grad_(True)
+    ids, w, aux, hist = B.forward_router(lg, K, use_sigmoid=sig, norm_expert_weight=norm, force_balance=True)
+    assert torch.equal(ids.cpu(), ref_ids) and torch.equal(hist.cpu(), ref_hist)
+    assert rel_l2(w, ref_w) <= 1e-5 and abs(float(aux) - float(ref_aux)) <= 1e-4 * abs(float(ref_aux))
+    gw = torch.randn(T, K, generator=gen)
+    (ref_w * gw).sum().backward()
+    (w * gw.to(DEV)).sum().backward()
+    assert rel_l2(lg.grad, lr.grad) <= 1e-4
+    if E <= 512:  # the same switch with the gate GEMM in front
+        x = _grid((T, 64), gen, steps=16)
+        wg = _grid((E, 64), gen, steps=16)
+        ids2, _w2, _aux2, hist2 = B.forward_gate_router(
+            x.bfloat16().to(DEV), wg.bfloat16().to(DEV), K, fp32_output=True, use_sigmoid=sig, norm_expert_weight=norm,
+            force_balance=True,
+        )
+        assert torch.equal(ids2.cpu(), ref_ids) and torch.equal(hist2.cpu(), ref_hist)
+
+
 # ------------------------------------------------------------------ whole layer, reduced configs
 @pytest.mark.parametrize(
     "name,T,E,tol",

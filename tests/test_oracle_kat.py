@@ -318,3 +318,15 @@ def test_balance_bias_update_closed_form():
     assert torch.equal(out, torch.tensor([0.375, -0.125, 0.0, 1.0]))
     # the update never changes the sum when loads are symmetric about the mean
     assert float(O.update_router_balance_bias(torch.tensor([3, 1]), torch.zeros(2), 1.0).sum()) == 0.0
+
+
+def test_router_force_balance_rule():
+    # reference moe_block.py:249-256: round-robin ids over the flat slots, equal counts when E divides T*K
+    logits = torch.randn(12, 6, generator=torch.Generator().manual_seed(0))
+    ids, w, aux, hist = O.forward_router(logits, 3, force_balance=True)
+    assert ids.flatten().tolist() == [i % 6 for i in range(36)] and hist.tolist() == [6] * 6
+    prob = torch.softmax(logits, 1)
+    assert torch.allclose(w, prob.gather(1, ids) / prob.gather(1, ids).sum(1, keepdim=True))
+    assert abs(float(aux) - 36.0) < 1e-4  # sum_e mean_t(p) * 6 * E = 6 * 6 * sum_e mean_t p = 36
+    with pytest.raises(ValueError):
+        O.forward_router(logits, 7, force_balance=True)
