@@ -81,14 +81,17 @@ def grouped_gemm_fp8_pow2(a_codes, a_scales, b_codes, b_scales, batch_sizes, out
     return out
 
 
-def grouped_gemm_fp8_pow2_rows(a_codes, a_scales, b_codes, b_scales, offsets, out_dtype) -> torch.Tensor:
+def grouped_gemm_fp8_pow2_rows(a_codes, a_scales, b_codes, b_scales, offsets, out_dtype, zero_tail=True) -> torch.Tensor:
     """:func:`grouped_gemm_fp8_pow2` for callers that hold the int32 row offsets ``[G+1]`` on the
-    device already (no host round trip); rows past the last group stay zero."""
+    device already (no host round trip); rows past the last group stay zero, or, with
+    ``zero_tail=False``, keep whatever the buffer held (for callers that never read them: saves
+    a fill of the whole output)."""
     from steptronoss_amd.model.utils.moe_utils import _gemm_workspace
 
     m_cap, k = a_codes.shape
     n_groups, n, _ = b_codes.shape
-    out = torch.zeros((m_cap, n), device=a_codes.device, dtype=out_dtype)
+    alloc = torch.zeros if zero_tail else torch.empty
+    out = alloc((m_cap, n), device=a_codes.device, dtype=out_dtype)
     ws = _gemm_workspace(m_cap, n_groups, a_codes.device)
     call(
         "stm_grouped_gemm_fp8_pow2", ptr(a_codes), ptr(a_scales), ptr(b_codes), ptr(b_scales), ptr(out), ptr(offsets),

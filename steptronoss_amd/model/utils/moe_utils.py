@@ -937,17 +937,24 @@ class _Fp8RoutedFFN(torch.autograd.Function):
             elif settings.deferred_id_check:
                 _defer_status_check(status)
             live = offsets[E:]
-            xp = torch.zeros((n_rows, H), device=dev, dtype=x.dtype)  # (unused rows are quantised too: keep them finite)
-            call("stm_permute_fwd", ptr(x), ptr(pos), 0, ptr(xp), T, K, H * x.element_size(), n_rows, None, stream())
-            q, sc = quantize_e4m3_1x128_pow2(xp)
-            gu = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w1_q, ffn.w1_s, offsets, x.dtype)
+            # Quantisation is row-local, so the T token rows are quantised once and their codes
+            # (one byte per element) and scales are moved to expert order, instead of permuting the
+            # 16-bit rows and quantising all T*K copies: the same codes and scales, bit for bit.
+            # (Rows of unused slots keep whatever the buffers held: no GEMM tile reads them.)
+            qx, sx = quantize_e4m3_1x128_pow2(x.contiguous())
+            token_of_row = torch.zeros(n_rows, device=dev, dtype=torch.int32)
+            call("stm_slot_tokens_to_rows", ptr(pos), n_rows, K, ptr(token_of_row), n_rows, stream())
+            q = torch.empty((n_rows, H), device=dev, dtype=torch.uint8)
+            call("stm_permute_fwd", ptr(qx), ptr(pos), 0, ptr(q), T, K, H, n_rows, None, stream())
+            sc = sx.index_select(1, token_of_row)
+            gu = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w1_q, ffn.w1_s, offsets, x.dtype, zero_tail=False)
             h = swiglu_fwd_rows(gu, swiglu_limit, live)
             q, sc = quantize_e4m3_1x128_pow2(h)
-            y = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w2_q, ffn.w2_s, offsets, x.dtype)
+            y = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w2_q, ffn.w2_s, offsets, x.dtype, zero_tail=False)
             addend = None if out_addend is None else out_addend.contiguous()
             out = _combine_rows(y, pos, token_weights, out_scale, addend)
             _nothing_routed_fwd(live, x, token_weights, out, out_scale, addend)
-        ctx.save_for_backward(w1, w2, x, xp, gu, h, y, pos, offsets, token_weights)
+        ctx.save_for_backward(w1, w2, x, gu, h, y, pos, offsets, token_weights)
         ctx.ffn = ffn
         ctx.limit = swiglu_limit
         ctx.out_scale = out_scale
@@ -959,7 +966,7 @@ class _Fp8RoutedFFN(torch.autograd.Function):
         from steptronoss_amd.model.common.feed_forward import swiglu_bwd_rows
         from steptronoss_amd.model.utils.fp8 import grouped_gemm_fp8_pow2_rows, quantize_e4m3_1x128_pow2
 
-        w1, w2, x, xp, gu, h, y, pos, offsets, token_weights = ctx.saved_tensors
+        w1, w2, x, gu, h, y, pos, offsets, token_weights = ctx.saved_tensors
         T, H, K, E = ctx.shape
         ffn = ctx.ffn
         dev = grad_out.device
@@ -968,19 +975,22 @@ class _Fp8RoutedFFN(torch.autograd.Function):
         with torch.cuda.device(dev):
             live = offsets[E:]
             go = grad_out.contiguous()
-            gy = torch.zeros_like(y)
+            gy = torch.empty_like(y)  # (rows of unused slots are never read)
             gtw = _combine_rows_bwd(go, y, pos, token_weights, gy, None, ctx.out_scale)
             if need_w2:
                 gw2 = _gemm_wgrad(gy, h, offsets, E)
             if need_w1 or need_x:
                 q, sc = quantize_e4m3_1x128_pow2(gy)
-                dh = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w2t_q, ffn.w2t_s, offsets, gy.dtype)
+                dh = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w2t_q, ffn.w2t_s, offsets, gy.dtype, zero_tail=False)
                 dgu = swiglu_bwd_rows(gu, dh, ctx.limit, live)
-                if need_w1:
-                    gw1 = _gemm_wgrad(dgu, xp, offsets, E)
+                if need_w1:  # (bf16 weight gradient: the token rows gathered in the GEMM loads, or copied first)
+                    if _gathered_takes(x):
+                        gw1 = _gemm_wgrad_gathered(dgu, x, offsets, E, _token_of_row(pos, K), 2)
+                    if gw1 is None:
+                        gw1 = _gemm_wgrad(dgu, _permuted_rows(x, pos, K), offsets, E)
                 if need_x:
                     q, sc = quantize_e4m3_1x128_pow2(dgu)
-                    dxp = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w1t_q, ffn.w1t_s, offsets, gy.dtype)
+                    dxp = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w1t_q, ffn.w1t_s, offsets, gy.dtype, zero_tail=False)
                     gx = _permute_rows_bwd(dxp, pos, H)
             if need_x or need_tw:
                 _nothing_routed_bwd(live, go, x, token_weights, gx, gtw if need_tw else None, ctx.out_scale)
