@@ -54,6 +54,7 @@ enum {
   STM_ST_NOT_INJECTIVE = 4,   /* two slots name the same row                              */
   STM_ST_ROW_OUT_OF_RANGE = 5, /* a pos >= n_rows was seen                                 */
   STM_ST_MAX_ROW_PLUS1 = 6,   /* 1 + the largest pos seen by stm_index_check (0 if none)  */
+  STM_ST_MAX_COUNT = 7,       /* slots of the expert with the most (routing kernels)      */
   STM_STATUS_WORDS = 8
 };
 

@@ -25,7 +25,8 @@ STM_F32, STM_F16, STM_BF16 = 0, 1, 2
     ST_NOT_INJECTIVE,
     ST_ROW_OUT_OF_RANGE,
     ST_MAX_ROW_PLUS1,
-) = range(7)
+    ST_MAX_COUNT,
+) = range(8)
 STATUS_WORDS = 8
 
 _DTYPE_CODE = {torch.float32: STM_F32, torch.float16: STM_F16, torch.bfloat16: STM_BF16}

@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(int32_t* __restrict_
   }
   __syncthreads();
   // per expert: totals over the slices, slices -> exclusive prefixes
-  int32_t sum_actual = 0;
+  int32_t sum_actual = 0, max_actual = 0;
   for (int e = tid; e < n_experts; e += kScanThreads) {
     int32_t run = 0;
     for (int gg = 0; gg < groups; ++gg) {
@@ -159,6 +159,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(int32_t* __restrict_
     }
     if (hist_out) hist_out[e] = run;
     sum_actual += run;
+    max_actual = run > max_actual ? run : max_actual;
     int32_t b = run;
     if (given) {
       if constexpr (GIVEN_I64) {
@@ -175,17 +176,24 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(int32_t* __restrict_
   __syncthreads();
   // number of valid slots (sum of the actual counts) via a throw-away scan
   __shared__ int32_t per_thread[kScanThreads];
+  __shared__ int32_t per_thread_max[kScanThreads];
   per_thread[tid] = sum_actual;
+  per_thread_max[tid] = max_actual;
   __syncthreads();
-  int32_t n_valid = 0;
+  int32_t n_valid = 0, largest = 0;
   if (tid < kWave) {
-    int32_t acc = 0;
-    for (int i = tid; i < kScanThreads; i += kWave) acc += per_thread[i];
+    int32_t acc = 0, most = 0;
+    for (int i = tid; i < kScanThreads; i += kWave) {
+      acc += per_thread[i];
+      most = per_thread_max[i] > most ? per_thread_max[i] : most;
+    }
     n_valid = wave_sum(acc);
+    largest = wave_max(most);
   }
   const int32_t given_total = block_exclusive_scan(base, n_experts, wave_sums);
   if (tid == 0) {
     status[STM_ST_N_VALID] = n_valid;
+    status[STM_ST_MAX_COUNT] = largest;
     if (given && given_total != n_valid) status[STM_ST_HIST_MISMATCH] = 1;
     if (flags[0]) status[STM_ST_HIST_NEGATIVE] = 1;
   }

@@ -73,7 +73,10 @@ class Settings:
         permuted copy of ``x`` (reference ``moe_scatter``, moe_utils.py:226) nor of ``grad_out``: the
         GEMMs that read those rows (forward 1, both weight gradients, the input gradient of GEMM 2)
         gather them through a row -> token table in their loads.  Off, or for a shape those kernels
-        do not take: the rows are copied first, as before.
+        do not take: the rows are copied first, as before.  With ``True`` the two weight gradients
+        fall back to copied rows while the routing is skewed (largest expert above three times
+        the mean in the latest status words that have arrived; see ``_wgrad_gathers``);
+        ``"all"`` gathers regardless.
     deferred_id_check: ``routed_grouped_ffn`` copies the routing status words to pinned host
         memory without waiting; a later call (or ``check_deferred_status()``) that finds such a
         copy complete raises the reference's "out-of-range" ``ValueError`` for an expert id
@@ -88,7 +91,7 @@ class Settings:
     deferred_id_check: bool = True
     fp8_experts: bool = False
     fuse_gate: bool | str = True
-    gather_in_gemm: bool = True
+    gather_in_gemm: bool | str = True
 
 
 settings = Settings()
@@ -181,13 +184,29 @@ def hip_index_compute(indices: torch.Tensor, expert_histogram: torch.Tensor) -> 
 _PENDING_STATUS: collections.deque = collections.deque()
 
 
-def _defer_status_check(status: torch.Tensor) -> None:
+_LAST_LOAD = {"skew": None}  # largest expert's slots over the mean, from the newest status copy that has arrived
+
+
+def _defer_status_check(status: torch.Tensor, n_experts: int = 0) -> None:
     """Start an asynchronous copy of the status words to pinned host memory; nothing waits."""
     host = torch.empty(status.shape, dtype=status.dtype, pin_memory=True)
     host.copy_(status, non_blocking=True)
     done = torch.cuda.Event()
     done.record()
-    _PENDING_STATUS.append((done, host))
+    _PENDING_STATUS.append((done, host, n_experts))
+
+
+def _wgrad_gathers() -> bool:
+    """Whether the weight gradients gather the token rows in their loads.  They do for
+    ``gather_in_gemm="all"``, and for ``True`` unless the routing of the latest call whose status
+    words have arrived was skewed (largest expert above three times the mean): the gathered
+    weight gradient pays per contraction step, which a long hot expert turns into the critical
+    path, so skewed loads copy the rows first.  (The information is one or more calls old by
+    design: nothing on the path waits for it.)"""
+    if settings.gather_in_gemm == "all":
+        return True
+    skew = _LAST_LOAD["skew"]
+    return bool(settings.gather_in_gemm) and (skew is None or skew <= 3.0)
 
 
 def check_deferred_status(wait: bool = False) -> None:
@@ -196,13 +215,15 @@ def check_deferred_status(wait: bool = False) -> None:
     one of them saw an expert id ``>= E``."""
     bad = False
     while _PENDING_STATUS:
-        done, host = _PENDING_STATUS[0]
+        done, host, n_experts = _PENDING_STATUS[0]
         if wait:
             done.synchronize()
         elif not done.query():
             break
         _PENDING_STATUS.popleft()
         bad = bad or bool(host[_lib.ST_ID_OUT_OF_RANGE])
+        if n_experts > 0 and int(host[_lib.ST_N_VALID]) > 0:
+            _LAST_LOAD["skew"] = int(host[_lib.ST_MAX_COUNT]) * n_experts / int(host[_lib.ST_N_VALID])
     if bad:
         _PENDING_STATUS.clear()
         raise ValueError("top_k_rank contains out-of-range expert index")
@@ -781,7 +802,7 @@ class _FusedRoutedFFN(torch.autograd.Function):
                 if int(status[_lib.ST_ID_OUT_OF_RANGE]):
                     raise ValueError("top_k_rank contains out-of-range expert index")
             elif settings.deferred_id_check:
-                _defer_status_check(status)
+                _defer_status_check(status, E)
             live = offsets[E:]  # device word: number of used rows
             w_row = None
             if settings.weights_before_gemm2 and token_weights.dtype == torch.float32:
@@ -862,7 +883,7 @@ class _FusedRoutedFFN(torch.autograd.Function):
                             dtype_code(gtw.dtype), stream(),
                         )  # fmt: skip
                 if need_w2:
-                    if gy is None and gathered_go and not _takes_main_grad(w2):
+                    if gy is None and gathered_go and _wgrad_gathers() and not _takes_main_grad(w2):
                         gw2 = _gemm_wgrad_gathered(go, h, offsets, E, token_of_row, 1)
                     if gw2 is None and gy is None:
                         gy = _permuted_rows(go, pos, K)
@@ -879,7 +900,7 @@ class _FusedRoutedFFN(torch.autograd.Function):
                     dh = _gemm_rows(gy, w2, offsets, h.shape[1], False)
                     dgu = swiglu_bwd_rows(gu, dh, ctx.limit, live)
                 if need_w1:
-                    if xp is None and not _takes_main_grad(w1):
+                    if xp is None and _wgrad_gathers() and not _takes_main_grad(w1):
                         gw1 = _gemm_wgrad_gathered(dgu, x, offsets, E, token_of_row, 2)
                     if gw1 is None:
                         if xp is None:
@@ -935,7 +956,7 @@ class _Fp8RoutedFFN(torch.autograd.Function):
                 if int(status[_lib.ST_ID_OUT_OF_RANGE]):
                     raise ValueError("top_k_rank contains out-of-range expert index")
             elif settings.deferred_id_check:
-                _defer_status_check(status)
+                _defer_status_check(status, E)
             live = offsets[E:]
             # Quantisation is row-local, so the T token rows are quantised once and their codes
             # (one byte per element) and scales are moved to expert order, instead of permuting the
@@ -984,7 +1005,7 @@ class _Fp8RoutedFFN(torch.autograd.Function):
                 dh = grouped_gemm_fp8_pow2_rows(q, sc, ffn.w2t_q, ffn.w2t_s, offsets, gy.dtype, zero_tail=False)
                 dgu = swiglu_bwd_rows(gu, dh, ctx.limit, live)
                 if need_w1:  # (bf16 weight gradient: the token rows gathered in the GEMM loads, or copied first)
-                    if _gathered_takes(x):
+                    if _gathered_takes(x) and _wgrad_gathers():
                         gw1 = _gemm_wgrad_gathered(dgu, x, offsets, E, _token_of_row(pos, K), 2)
                     if gw1 is None:
                         gw1 = _gemm_wgrad(dgu, _permuted_rows(x, pos, K), offsets, E)

@@ -272,7 +272,7 @@ def test_ffn_gathers_token_rows_in_the_gemm_loads(weights_before_gemm2, dtype, i
         finally:
             M.settings.gather_in_gemm = old
 
-    gathered, ran = run(True)
+    gathered, ran = run("all")
     copied, ran_copied = run(False)
     assert "stm_permute_fwd" in ran_copied and "stm_grouped_gemm_swiglu_gathered" not in ran_copied
     assert "stm_permute_fwd" not in ran
@@ -286,6 +286,44 @@ def test_ffn_gathers_token_rows_in_the_gemm_loads(weights_before_gemm2, dtype, i
     assert rel_l2(gathered[0], ref) <= BF16_TOL
     for got, r in zip(gathered[1:], ref_in):
         assert rel_l2(got, r.grad) <= BF16_TOL
+
+
+def test_ffn_weight_gradients_copy_their_rows_while_the_routing_is_skewed():
+    # gather_in_gemm=True: forward 1 and the input gradient of GEMM 2 always gather; the two
+    # weight gradients do unless the latest routing status that has arrived shows a hot expert
+    from steptronoss_amd.profiling import KernelTimer
+
+    gen = torch.Generator().manual_seed(22)
+    T, H, K, E, Fh = 2048, 512, 4, 8, 256
+    x = (torch.randn(T, H, generator=gen) * 0.5).bfloat16()
+    w1 = (torch.randn(E, 2 * Fh, H, generator=gen) * 0.05).bfloat16()
+    w2 = (torch.randn(E, H, Fh, generator=gen) * 0.05).bfloat16()
+    ids = make_topk_ids(T, K, E, gen=gen).to(DEV)
+    tw = torch.rand(T, K, generator=gen)
+    go = torch.randn(T, H, generator=gen).bfloat16().to(DEV)
+    old = (M.settings.gather_in_gemm, M._LAST_LOAD["skew"])
+    results = {}
+    try:
+        M.settings.gather_in_gemm = True
+        for skew in (1.1, 10.0):
+            M.check_deferred_status(wait=True)  # (so that no older status copy overwrites the figure set here)
+            M._LAST_LOAD["skew"] = skew
+            ins = [t.to(DEV).requires_grad_(True) for t in (w1, w2, x, tw)]
+            with KernelTimer() as kt:
+                out = M.routed_grouped_ffn(ins[0], ins[1], swiglu, ins[2], ids, ins[3])
+                M._LAST_LOAD["skew"] = skew  # (the call itself may have harvested a newer status)
+                out.backward(go)
+            ran = set(kt.summary())
+            assert {"stm_grouped_gemm_swiglu_gathered", "stm_grouped_gemm_dswiglu_gathered"} <= ran
+            assert ("stm_grouped_gemm_wgrad_gathered" in ran) == (skew < 3) and ("stm_permute_fwd" in ran) == (skew > 3)
+            results[skew] = [out.detach()] + [t.grad for t in ins]
+        for a, b in zip(results[1.1], results[10.0]):
+            assert torch.equal(a, b)
+        # and the status words do carry the figure: the uniform routing above is far from skewed
+        M.check_deferred_status(wait=True)
+        assert 1.0 <= M._LAST_LOAD["skew"] < 1.5
+    finally:
+        M.settings.gather_in_gemm, M._LAST_LOAD["skew"] = old
 
 
 def test_slot_and_row_order_helpers():
