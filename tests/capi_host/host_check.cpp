@@ -6,10 +6,13 @@
 //   route plan  -> histogram, offsets and positions of a stable counting sort (integers, exact)
 //   permute     -> rows copied to their positions (exact)
 //   grouped GEMM-> fp32, every group against a triple loop (1e-5 relative)
+//   gathered weight gradient (bf16) -> the product read through the row -> token table against
+//                  the same product on copied rows (bit for bit) and a host loop (1e-2 relative)
 #include <hip/hip_runtime_api.h>
 #include <math.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <string.h>
 #include <vector>
 
 #include "../../include/steptron_moe.h"
@@ -32,6 +35,18 @@ namespace {
       return 2;                                                                      \
     }                                                                                \
   } while (0)
+
+uint16_t to_bf16(float f) {  // round to nearest even
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return uint16_t((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+float from_bf16(uint16_t h) {
+  const uint32_t u = uint32_t(h) << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
 
 template <typename T>
 struct DeviceBuffer {
@@ -131,6 +146,81 @@ extern "C" int stm_host_check(char* msg, int cap) {
           return 5;
         }
       }
+  // weight gradient with a gathered operand, bf16: out[g] = d[rows of g]^T @ tokens[token_of_row[rows of g]]
+  {
+    const int T2 = 512, K2 = 2, E2 = 4, P = 256, Q = 256;
+    const int64_t slots2 = int64_t(T2) * K2;
+    std::vector<int32_t> ids2(slots2);
+    for (auto& v : ids2) {
+      state = state * 1664525u + 1013904223u;
+      v = int32_t((state >> 9) % uint32_t(E2));
+    }
+    std::vector<int32_t> off2(E2 + 1, 0), pos2(slots2), nxt(E2, 0);
+    for (int32_t e : ids2) ++off2[e + 1];
+    for (int e = 0; e < E2; ++e) off2[e + 1] += off2[e];
+    for (int e = 0; e < E2; ++e) nxt[e] = off2[e];
+    for (int64_t i = 0; i < slots2; ++i) pos2[i] = nxt[ids2[i]]++;
+    std::vector<uint16_t> tok(size_t(T2) * Q), d(size_t(slots2) * P);
+    for (size_t i = 0; i < tok.size(); ++i) tok[i] = to_bf16(float(int((i * 7u) % 31u) - 15) * 0.0625f);
+    for (size_t i = 0; i < d.size(); ++i) d[i] = to_bf16(float(int((i * 5u) % 23u) - 11) * 0.125f);
+    DeviceBuffer<int32_t> d_ids2, d_hist2, d_off2, d_pos2, d_st2, d_table;
+    DeviceBuffer<unsigned char> d_ws2;
+    DeviceBuffer<uint16_t> d_tok, d_d, d_copy, d_out_g, d_out_c;
+    const size_t ws2 = stm_route_workspace_bytes(slots2, E2);
+    CHECK_HIP(d_ids2.alloc(slots2));
+    CHECK_HIP(d_hist2.alloc(E2));
+    CHECK_HIP(d_off2.alloc(E2 + 1));
+    CHECK_HIP(d_pos2.alloc(slots2));
+    CHECK_HIP(d_st2.alloc(STM_STATUS_WORDS));
+    CHECK_HIP(d_ws2.alloc(ws2));
+    CHECK_HIP(d_table.alloc(size_t(slots2) + size_t(stm_row_sources_padding())));
+    CHECK_HIP(d_tok.alloc(tok.size()));
+    CHECK_HIP(d_d.alloc(d.size()));
+    CHECK_HIP(d_copy.alloc(size_t(slots2) * Q));
+    CHECK_HIP(d_out_g.alloc(size_t(E2) * P * Q));
+    CHECK_HIP(d_out_c.alloc(size_t(E2) * P * Q));
+    CHECK_HIP(hipMemcpy(d_ids2.p, ids2.data(), slots2 * sizeof(int32_t), hipMemcpyHostToDevice));
+    CHECK_HIP(hipMemcpy(d_tok.p, tok.data(), tok.size() * 2, hipMemcpyHostToDevice));
+    CHECK_HIP(hipMemcpy(d_d.p, d.data(), d.size() * 2, hipMemcpyHostToDevice));
+    CHECK_HIP(hipMemset(d_st2.p, 0, STM_STATUS_WORDS * sizeof(int32_t)));
+    CHECK_STM(stm_route_plan(d_ids2.p, 0, slots2, E2, d_hist2.p, d_off2.p, d_pos2.p, d_st2.p, d_ws2.p, ws2, nullptr));
+    CHECK_STM(stm_slot_tokens_to_rows(d_pos2.p, slots2, K2, d_table.p, slots2, nullptr));
+    CHECK_STM(stm_grouped_gemm_wgrad_gathered(d_d.p, d_tok.p, d_out_g.p, d_off2.p, E2, slots2, P, Q, STM_BF16, d_table.p, 2,
+                                              T2, nullptr));
+    CHECK_STM(stm_permute_fwd(d_tok.p, d_pos2.p, 0, d_copy.p, T2, K2, int64_t(Q) * 2, slots2, nullptr, nullptr));
+    CHECK_STM(stm_grouped_gemm_wgrad(d_d.p, d_copy.p, d_out_c.p, d_off2.p, E2, slots2, P, Q, STM_BF16, nullptr));
+    CHECK_HIP(hipDeviceSynchronize());
+    std::vector<int32_t> st2(STM_STATUS_WORDS);
+    CHECK_HIP(hipMemcpy(st2.data(), d_st2.p, st2.size() * sizeof(int32_t), hipMemcpyDeviceToHost));
+    int largest = 0;
+    for (int e = 0; e < E2; ++e) largest = off2[e + 1] - off2[e] > largest ? off2[e + 1] - off2[e] : largest;
+    if (st2[STM_ST_N_VALID] != int32_t(slots2) || st2[STM_ST_MAX_COUNT] != largest) {
+      snprintf(msg, cap, "status words: %d valid, largest %d; expected %d, %d", st2[STM_ST_N_VALID], st2[STM_ST_MAX_COUNT],
+               int(slots2), largest);
+      return 6;
+    }
+    std::vector<uint16_t> out_g(size_t(E2) * P * Q), out_c(out_g.size());
+    CHECK_HIP(hipMemcpy(out_g.data(), d_out_g.p, out_g.size() * 2, hipMemcpyDeviceToHost));
+    CHECK_HIP(hipMemcpy(out_c.data(), d_out_c.p, out_c.size() * 2, hipMemcpyDeviceToHost));
+    if (out_g != out_c) {
+      snprintf(msg, cap, "gathered weight gradient differs from the one on copied rows");
+      return 7;
+    }
+    std::vector<int32_t> token_of(slots2);
+    for (int64_t i = 0; i < slots2; ++i) token_of[pos2[i]] = int32_t(i / K2);
+    for (int e = 0; e < E2; ++e)
+      for (int pi = 0; pi < P; pi += 37)
+        for (int qi = 0; qi < Q; qi += 41) {
+          double ref = 0.0;
+          for (int r = off2[e]; r < off2[e + 1]; ++r)
+            ref += double(from_bf16(d[size_t(r) * P + pi])) * double(from_bf16(tok[size_t(token_of[r]) * Q + qi]));
+          const double got = from_bf16(out_g[(size_t(e) * P + pi) * Q + qi]);
+          if (fabs(got - ref) > 1e-2 * (fabs(ref) + 1.0)) {
+            snprintf(msg, cap, "gathered weight gradient: expert %d [%d, %d] is %g, expected %g", e, pi, qi, got, ref);
+            return 8;
+          }
+        }
+  }
   snprintf(msg, cap, "ok: %d slots, %d rows, %d experts (abi %d)", int(n_slots), n_rows, E, stm_abi_version());
   return 0;
 }

@@ -1,6 +1,6 @@
 """The C ABI from a host that is not Python: ``tests/capi_host/host_check.cpp`` allocates its own
 device memory with the HIP runtime, calls the library through ``include/steptron_moe.h`` only and
-checks route plan, permute and grouped GEMM against loops on the host.  It is built (by
+checks route plan, permute, grouped GEMM and the gathered weight gradient against loops on the host.  It is built (by
 ``__graft_entry__.build()``) as a one-function shared library so that it can run inside this
 process; torch does not take part."""
 
